@@ -1,0 +1,135 @@
+/* maester_attn.h -- C ABI of the MI355X (gfx950) packed-SFT document-masked attention path.
+ *
+ * The library replaces, for maester's Gemma attention, everything between the qkv split and
+ * o_proj (maester/models/gemma/model.py:364-439) plus the per-step BlockMask construction
+ * (model.py:694-730).  The reference is pure Python on torch, so there is no FFI to mirror; each
+ * entry point below cites the reference code it stands in for.
+ *
+ * Conventions
+ *  - Every pointer is a DEVICE pointer owned by the caller (torch); the library allocates nothing,
+ *    never synchronises and never throws.  Work is enqueued on `stream` (a hipStream_t passed as
+ *    void*; NULL = the default stream).
+ *  - Every function returns MA_OK (0) or a negative MA_ERR_* code; the message of the last error of
+ *    the calling thread is available from ma_last_error().  Arguments are validated before any
+ *    launch, so the error paths run on a host without a GPU.
+ *  - Activations are addressed as x[b, s, h, d] = base + b*stride_b + s*stride_s + h*stride_h + d
+ *    (strides in ELEMENTS, last dim contiguous), which covers both the [B,S,H,D] views of the fused
+ *    qkv projection output (model.py:358-364) and [B,H,S,D] tensors.
+ *  - Tile lists use torch's BlockMask format with 128x128 tiles and a head dim of 1:
+ *    *_num_blocks int32 [B, T], *_indices int32 [B, T, T], T = ceil(S/128).
+ */
+#ifndef MAESTER_ATTN_H
+#define MAESTER_ATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MA_OK 0
+#define MA_ERR_BAD_ARG (-1)
+#define MA_ERR_UNSUPPORTED (-2)
+#define MA_ERR_LAUNCH (-3)
+
+#define MA_DTYPE_F32 0
+#define MA_DTYPE_BF16 1
+
+#define MA_TILE 128 /* BlockMask tile edge (torch _DEFAULT_SPARSE_BLOCK_SIZE) */
+
+/* Library version (major*10000 + minor*100 + patch). */
+int ma_version(void);
+
+/* Message describing the last error returned to the calling thread ("" if none). */
+const char* ma_last_error(void);
+
+/* Strided [B,S,H,D] activation descriptor (strides in elements). */
+typedef struct ma_tensor4 {
+    void* ptr;
+    int64_t stride_b, stride_s, stride_h;
+} ma_tensor4;
+
+/* The eight BlockMask tensors (torch/nn/attention/flex_attention.py BlockMask). */
+typedef struct ma_tile_map {
+    int32_t* kv_num_blocks;      /* [B,T]   partial tiles per q-tile row            */
+    int32_t* kv_indices;         /* [B,T,T] partial kv tiles ascending, then the rest */
+    int32_t* full_kv_num_blocks; /* [B,T]   full tiles per q-tile row               */
+    int32_t* full_kv_indices;    /* [B,T,T]                                          */
+    int32_t* q_num_blocks;       /* [B,T]   the same four on the transposed tile matrix */
+    int32_t* q_indices;          /* [B,T,T]                                          */
+    int32_t* full_q_num_blocks;  /* [B,T]                                            */
+    int32_t* full_q_indices;     /* [B,T,T]                                          */
+} ma_tile_map;
+
+/* ---- block-sparse tile map --------------------------------------------------------------------
+ * Replaces create_block_mask(make_document_mask_wrapper(base, document_ids), B, None, S, S)
+ * (maester/models/gemma/model.py:694-706 global, 714-730 local; torch
+ * flex_attention.py:979-1022 tile counts, 429-441 ordered lists).  Predicate:
+ *   same_doc(q,kv) && (!causal || q >= kv) && (window < 0 || (q >= kv && q - kv <= window)).
+ * document_ids: int64 [B,S] contiguous, or NULL (no document term; model.py:227-228).
+ * workspace: at least ma_tile_map_workspace_bytes(B,S) bytes of device scratch.
+ * Output is bit-exact with torch's BlockMask tensors, including the list tails. */
+size_t ma_tile_map_workspace_bytes(int B, int S);
+int ma_tile_map_build(const int64_t* document_ids, int B, int S, int causal, int64_t window,
+                      const ma_tile_map* out, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- fused QK-RMSNorm + RoPE prologue ------------------------------------------------------------
+ * Replaces query_norm/key_norm (model.py:135-172, 366-368) followed by apply_rotary_emb
+ * (model.py:97-106, 371-372) with the table gather by position_ids (model.py:744-747):
+ *   r = rsqrt(mean(x^2) + eps); y = x*r*(add_unit_offset ? 1+w : w);
+ *   out[:D/2] = y[:D/2]*cos - y[D/2:]*sin;  out[D/2:] = y[:D/2]*sin + y[D/2:]*cos   (fp32 math).
+ * q_weight/k_weight: fp32 [D] stored parameters, or NULL for no norm (use_qk_norm=False).
+ * rope_cos/rope_sin: fp32 [n_pos, D/2].  position_ids: int64 [B,S] contiguous or NULL (= arange).
+ * q_rstd/k_rstd: fp32 [B,S,Hq]/[B,S,Hkv] outputs saved for the backward (may be NULL when the
+ * matching weight is NULL).  Input and output may alias. */
+int ma_prologue_fwd(const ma_tensor4* q_in, const ma_tensor4* k_in, const ma_tensor4* q_out,
+                    const ma_tensor4* k_out, const float* q_weight, const float* k_weight,
+                    const float* rope_cos, const float* rope_sin, int64_t n_pos,
+                    const int64_t* position_ids, float eps, int add_unit_offset, float* q_rstd,
+                    float* k_rstd, int dtype, int B, int S, int Hq, int Hkv, int D, void* stream);
+
+/* Backward of the prologue (autograd of the same reference lines).  dq_out/dk_out are the
+ * gradients w.r.t. the prologue outputs, dq_in/dk_in receive the gradients w.r.t. its inputs (may
+ * alias dq_out/dk_out).  dq_weight/dk_weight: fp32 [D] outputs (NULL with a NULL weight); they are
+ * reduced without atomics through `workspace` (ma_prologue_bwd_workspace_bytes). */
+size_t ma_prologue_bwd_workspace_bytes(int B, int S, int Hq, int Hkv, int D);
+int ma_prologue_bwd(const ma_tensor4* q_in, const ma_tensor4* k_in, const ma_tensor4* dq_out,
+                    const ma_tensor4* dk_out, const ma_tensor4* dq_in, const ma_tensor4* dk_in,
+                    const float* q_weight, const float* k_weight, const float* rope_cos,
+                    const float* rope_sin, int64_t n_pos, const int64_t* position_ids,
+                    int add_unit_offset, const float* q_rstd, const float* k_rstd, float* dq_weight,
+                    float* dk_weight, void* workspace, size_t workspace_bytes, int dtype, int B,
+                    int S, int Hq, int Hkv, int D, void* stream);
+
+/* ---- GQA flash-style attention ---------------------------------------------------------------------
+ * Replaces torch.compile(flex_attention)(q, k, v, block_mask, scale, enable_gqa)
+ * (model.py:384-396; torch/_higher_order_ops/flex_attention.py:159-267) with the output already in
+ * the [B,S,Hq,D] layout that model.py:436-438 produces by a transposed copy.
+ *   O = softmax(scale * Q K^T + mask) V, q head h reads kv head h / (Hq/Hkv).
+ * lse: fp32 [B,Hq,S] output, natural-log log-sum-exp of the scaled masked scores.
+ * map: tile lists from ma_tile_map_build for the SAME (document_ids, causal, window); only tiles in
+ * the kv lists are visited, elements of partial tiles are masked with the predicate above.
+ * D in {64,128,256}; Hq % Hkv == 0. */
+int ma_attn_fwd(const ma_tensor4* q, const ma_tensor4* k, const ma_tensor4* v, const ma_tensor4* out,
+                float* lse, const ma_tile_map* map, const int64_t* document_ids, int causal,
+                int64_t window, float scale, int dtype, int B, int S, int Hq, int Hkv, int D,
+                void* stream);
+
+/* Backward (torch/_higher_order_ops/flex_attention.py:825-993):
+ *   delta = rowsum(O * dO); P = exp(S - lse); dV = P^T dO; dS = P * (dO V^T - delta);
+ *   dQ = scale * dS K; dK = scale * dS^T Q; dK/dV summed over the Hq/Hkv query heads of a kv head.
+ * dK and dV are produced without global atomics (one workgroup owns a kv tile and walks the q-side
+ * lists), so results are run-to-run deterministic.
+ * workspace: ma_attn_bwd_workspace_bytes(...) bytes (holds delta, fp32 [B,Hq,S]). */
+size_t ma_attn_bwd_workspace_bytes(int B, int S, int Hq, int Hkv, int D);
+int ma_attn_bwd(const ma_tensor4* q, const ma_tensor4* k, const ma_tensor4* v, const ma_tensor4* out,
+                const ma_tensor4* dout, const float* lse, const ma_tensor4* dq, const ma_tensor4* dk,
+                const ma_tensor4* dv, const ma_tile_map* map, const int64_t* document_ids, int causal,
+                int64_t window, float scale, void* workspace, size_t workspace_bytes, int dtype,
+                int B, int S, int Hq, int Hkv, int D, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MAESTER_ATTN_H */

@@ -1,0 +1,253 @@
+"""``torch.autograd.Function`` front end of the HIP attention path.
+
+``PackedDocAttention`` takes what maester's ``GemmaAttention.forward`` holds right after the qkv
+split (maester/models/gemma/model.py:358-364) -- ``xq [B,S,Hq,D]``, ``xk/xv [B,S,Hkv,D]`` (strided
+views are fine), the stored QK-norm weights, RoPE tables, ``position_ids``, ``document_ids`` -- and
+returns the attention output in ``[B,S,Hq,D]``, i.e. model.py:366-438 in one call.  The two stages
+are also exposed on their own (``qk_norm_rope``, ``doc_masked_attention``).
+
+Everything runs in the HIP library; there is no PyTorch fallback.
+"""
+from __future__ import annotations
+
+from ctypes import byref
+
+import torch
+
+from . import _lib
+from .tile_map import TileMap, build_tile_map
+
+
+# ------------------------------------------------------------------------------------------------
+# raw stage wrappers (no autograd)
+# ------------------------------------------------------------------------------------------------
+def _check_qkv(xq, xk, xv=None):
+    if xq.dim() != 4 or xk.dim() != 4:
+        raise ValueError("expected [B,S,H,D] tensors")
+    B, S, Hq, D = xq.shape
+    if xk.shape[0] != B or xk.shape[1] != S or xk.shape[3] != D:
+        raise ValueError(f"q {tuple(xq.shape)} and k {tuple(xk.shape)} disagree")
+    if xv is not None and xv.shape != xk.shape:
+        raise ValueError(f"k {tuple(xk.shape)} and v {tuple(xv.shape)} disagree")
+    if xk.dtype != xq.dtype or (xv is not None and xv.dtype != xq.dtype):
+        raise TypeError("q, k, v must share one dtype")
+    return B, S, Hq, xk.shape[2], D
+
+
+def _rowmajor(t: torch.Tensor) -> torch.Tensor:
+    return t if t.stride(-1) == 1 else t.contiguous()
+
+
+def _ids(t: torch.Tensor | None, B: int, S: int, name: str):
+    if t is None:
+        return None
+    if tuple(t.shape) != (B, S):
+        raise ValueError(f"{name} shape {tuple(t.shape)} != {(B, S)}")
+    return t.detach().to(torch.long).contiguous()
+
+
+def prologue_forward(xq, xk, q_w, k_w, cos, sin, position_ids, eps=1e-6, add_unit_offset=True):
+    """Returns (q, k, q_rstd, k_rstd); q/k are new contiguous [B,S,H,D] tensors."""
+    _lib.require_gpu(xq, "prologue_forward")
+    B, S, Hq, Hkv, D = _check_qkv(xq, xk)
+    xq, xk = _rowmajor(xq), _rowmajor(xk)
+    dev = xq.device
+    q = torch.empty((B, S, Hq, D), dtype=xq.dtype, device=dev)
+    k = torch.empty((B, S, Hkv, D), dtype=xk.dtype, device=dev)
+    qw = None if q_w is None else q_w.detach().float().contiguous()
+    kw = None if k_w is None else k_w.detach().float().contiguous()
+    q_rstd = torch.empty((B, S, Hq), dtype=torch.float32, device=dev) if qw is not None else None
+    k_rstd = torch.empty((B, S, Hkv), dtype=torch.float32, device=dev) if kw is not None else None
+    pos = _ids(position_ids, B, S, "position_ids")
+    cos, sin = cos.contiguous(), sin.contiguous()
+    if cos.dtype != torch.float32 or cos.shape != sin.shape or cos.shape[-1] != D // 2:
+        raise ValueError(f"rope tables must be fp32 [P,{D // 2}], got {tuple(cos.shape)} {cos.dtype}")
+    with torch.cuda.device(dev):
+        rc = _lib.lib().ma_prologue_fwd(
+            byref(_lib.tensor4(xq)), byref(_lib.tensor4(xk)), byref(_lib.tensor4(q)), byref(_lib.tensor4(k)),
+            _lib.ptr(qw), _lib.ptr(kw), _lib.ptr(cos), _lib.ptr(sin), cos.shape[0], _lib.ptr(pos), float(eps),
+            1 if add_unit_offset else 0, _lib.ptr(q_rstd), _lib.ptr(k_rstd), _lib.dtype_code(xq.dtype), B, S, Hq,
+            Hkv, D, _lib.current_stream(dev))
+    _lib.check(rc)
+    return q, k, q_rstd, k_rstd
+
+
+def prologue_backward(xq, xk, dq, dk, q_w, k_w, cos, sin, position_ids, q_rstd, k_rstd, add_unit_offset=True,
+                      inplace=False):
+    """Gradients w.r.t. the prologue inputs: (dxq, dxk, dq_w fp32|None, dk_w fp32|None).
+    With ``inplace`` the incoming ``dq``/``dk`` buffers are overwritten with the result."""
+    B, S, Hq, Hkv, D = _check_qkv(dq, dk)
+    dev = dq.device
+    dq, dk = _rowmajor(dq), _rowmajor(dk)
+    dxq = dq if inplace else torch.empty((B, S, Hq, D), dtype=dq.dtype, device=dev)
+    dxk = dk if inplace else torch.empty((B, S, Hkv, D), dtype=dk.dtype, device=dev)
+    L = _lib.lib()
+    qw = None if q_w is None else q_w.detach().float().contiguous()
+    kw = None if k_w is None else k_w.detach().float().contiguous()
+    dqw = torch.empty(D, dtype=torch.float32, device=dev) if qw is not None else None
+    dkw = torch.empty(D, dtype=torch.float32, device=dev) if kw is not None else None
+    ws_bytes = L.ma_prologue_bwd_workspace_bytes(B, S, Hq, Hkv, D)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+    pos = _ids(position_ids, B, S, "position_ids")
+    xq_d = byref(_lib.tensor4(_rowmajor(xq))) if qw is not None else None
+    xk_d = byref(_lib.tensor4(_rowmajor(xk))) if kw is not None else None
+    with torch.cuda.device(dev):
+        rc = L.ma_prologue_bwd(
+            xq_d, xk_d, byref(_lib.tensor4(dq)), byref(_lib.tensor4(dk)), byref(_lib.tensor4(dxq)),
+            byref(_lib.tensor4(dxk)), _lib.ptr(qw), _lib.ptr(kw), _lib.ptr(cos), _lib.ptr(sin), cos.shape[0],
+            _lib.ptr(pos), 1 if add_unit_offset else 0, _lib.ptr(q_rstd), _lib.ptr(k_rstd), _lib.ptr(dqw),
+            _lib.ptr(dkw), _lib.ptr(ws), ws_bytes, _lib.dtype_code(dq.dtype), B, S, Hq, Hkv, D,
+            _lib.current_stream(dev))
+    _lib.check(rc)
+    return dxq, dxk, dqw, dkw
+
+
+def _resolve_map(tile_map, document_ids, B, S, causal, window, device) -> TileMap:
+    if tile_map is None:
+        return build_tile_map(document_ids, B, S, causal, window, device=device)
+    if tile_map.seq_len != S or tile_map.kv_num_blocks.shape[0] != B:
+        raise ValueError("tile_map was built for another batch/sequence shape")
+    if tile_map.causal != bool(causal) or tile_map.window != window:
+        raise ValueError("tile_map was built for another mask (causal/sliding_window)")
+    return tile_map
+
+
+def attention_forward(q, k, v, tile_map: TileMap, document_ids, scale, causal=True, window=None):
+    """Returns (out [B,S,Hq,D], lse [B,Hq,S] fp32)."""
+    _lib.require_gpu(q, "attention_forward")
+    B, S, Hq, Hkv, D = _check_qkv(q, k, v)
+    q, k, v = _rowmajor(q), _rowmajor(k), _rowmajor(v)
+    dev = q.device
+    out = torch.empty((B, S, Hq, D), dtype=q.dtype, device=dev)
+    lse = torch.empty((B, Hq, S), dtype=torch.float32, device=dev)
+    doc = _ids(document_ids, B, S, "document_ids")
+    cs = tile_map.c_struct()
+    with torch.cuda.device(dev):
+        rc = _lib.lib().ma_attn_fwd(
+            byref(_lib.tensor4(q)), byref(_lib.tensor4(k)), byref(_lib.tensor4(v)), byref(_lib.tensor4(out)),
+            _lib.ptr(lse), byref(cs), _lib.ptr(doc), 1 if causal else 0, -1 if window is None else int(window),
+            float(scale), _lib.dtype_code(q.dtype), B, S, Hq, Hkv, D, _lib.current_stream(dev))
+    _lib.check(rc)
+    return out, lse
+
+
+def attention_backward(q, k, v, out, dout, lse, tile_map: TileMap, document_ids, scale, causal=True, window=None):
+    """Returns (dq, dk, dv) as new contiguous [B,S,H,D] tensors."""
+    B, S, Hq, Hkv, D = _check_qkv(q, k, v)
+    q, k, v, out, dout = (_rowmajor(t) for t in (q, k, v, out, dout))
+    dev = q.device
+    L = _lib.lib()
+    dq = torch.empty((B, S, Hq, D), dtype=q.dtype, device=dev)
+    dk = torch.empty((B, S, Hkv, D), dtype=q.dtype, device=dev)
+    dv = torch.empty((B, S, Hkv, D), dtype=q.dtype, device=dev)
+    ws_bytes = L.ma_attn_bwd_workspace_bytes(B, S, Hq, Hkv, D)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+    doc = _ids(document_ids, B, S, "document_ids")
+    cs = tile_map.c_struct()
+    with torch.cuda.device(dev):
+        rc = L.ma_attn_bwd(
+            byref(_lib.tensor4(q)), byref(_lib.tensor4(k)), byref(_lib.tensor4(v)), byref(_lib.tensor4(out)),
+            byref(_lib.tensor4(dout)), _lib.ptr(lse), byref(_lib.tensor4(dq)), byref(_lib.tensor4(dk)),
+            byref(_lib.tensor4(dv)), byref(cs), _lib.ptr(doc), 1 if causal else 0,
+            -1 if window is None else int(window), float(scale), _lib.ptr(ws), ws_bytes,
+            _lib.dtype_code(q.dtype), B, S, Hq, Hkv, D, _lib.current_stream(dev))
+    _lib.check(rc)
+    return dq, dk, dv
+
+
+# ------------------------------------------------------------------------------------------------
+# autograd
+# ------------------------------------------------------------------------------------------------
+def _wgrad(g, w):
+    return None if (g is None or w is None) else g.to(w.dtype)
+
+
+class _QKNormRope(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, xq, xk, q_w, k_w, cos, sin, position_ids, eps, add_unit_offset):
+        q, k, q_rstd, k_rstd = prologue_forward(xq, xk, q_w, k_w, cos, sin, position_ids, eps, add_unit_offset)
+        ctx.save_for_backward(xq, xk, q_w, k_w, cos, sin, position_ids, q_rstd, k_rstd)
+        ctx.add_unit_offset = add_unit_offset
+        return q, k
+
+    @staticmethod
+    def backward(ctx, dq, dk):
+        xq, xk, q_w, k_w, cos, sin, position_ids, q_rstd, k_rstd = ctx.saved_tensors
+        dxq, dxk, dqw, dkw = prologue_backward(xq, xk, dq, dk, q_w, k_w, cos, sin, position_ids, q_rstd, k_rstd,
+                                               ctx.add_unit_offset)
+        return dxq, dxk, _wgrad(dqw, q_w), _wgrad(dkw, k_w), None, None, None, None, None
+
+
+class _DocMaskedAttention(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, document_ids, scale, causal, window, tile_map):
+        B, S = q.shape[0], q.shape[1]
+        tile_map = _resolve_map(tile_map, document_ids, B, S, causal, window, q.device)
+        out, lse = attention_forward(q, k, v, tile_map, document_ids, scale, causal, window)
+        ctx.save_for_backward(q, k, v, out, lse, document_ids)
+        ctx.tile_map, ctx.scale, ctx.causal, ctx.window = tile_map, scale, causal, window
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        q, k, v, out, lse, document_ids = ctx.saved_tensors
+        dq, dk, dv = attention_backward(q, k, v, out, dout, lse, ctx.tile_map, document_ids, ctx.scale, ctx.causal,
+                                        ctx.window)
+        return dq, dk, dv, None, None, None, None, None
+
+
+class PackedDocAttention(torch.autograd.Function):
+    """QK-RMSNorm -> RoPE -> document-masked GQA attention, forward and backward in HIP.
+
+    ``apply(xq, xk, xv, q_norm_w, k_norm_w, rope_cos, rope_sin, position_ids, document_ids, scale,
+    causal, sliding_window, eps, tile_map)`` -> ``out [B,S,Hq,D]`` (dtype of ``xq``).
+
+    ``q_norm_w`` / ``k_norm_w`` are the *stored* Gemma parameters (effective scale ``1 + w``,
+    maester/models/gemma/model.py:146,163-164) or ``None`` (``use_qk_norm=False``).  Gradients are
+    returned for xq, xk, xv and the two weights."""
+
+    @staticmethod
+    def forward(ctx, xq, xk, xv, q_norm_w, k_norm_w, rope_cos, rope_sin, position_ids, document_ids, scale,
+                causal=True, sliding_window=None, eps=1e-6, tile_map=None):
+        B, S = xq.shape[0], xq.shape[1]
+        tile_map = _resolve_map(tile_map, document_ids, B, S, causal, sliding_window, xq.device)
+        q, k, q_rstd, k_rstd = prologue_forward(xq, xk, q_norm_w, k_norm_w, rope_cos, rope_sin, position_ids, eps,
+                                                True)
+        out, lse = attention_forward(q, k, xv, tile_map, document_ids, scale, causal, sliding_window)
+        ctx.save_for_backward(xq, xk, xv, q_norm_w, k_norm_w, rope_cos, rope_sin, position_ids, document_ids, q, k,
+                              out, lse, q_rstd, k_rstd)
+        ctx.tile_map, ctx.scale, ctx.causal, ctx.window = tile_map, scale, causal, sliding_window
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        (xq, xk, xv, q_w, k_w, cos, sin, position_ids, document_ids, q, k, out, lse, q_rstd,
+         k_rstd) = ctx.saved_tensors
+        dq, dk, dv = attention_backward(q, k, xv, out, dout, lse, ctx.tile_map, document_ids, ctx.scale, ctx.causal,
+                                        ctx.window)
+        dxq, dxk, dqw, dkw = prologue_backward(xq, xk, dq, dk, q_w, k_w, cos, sin, position_ids, q_rstd, k_rstd, True,
+                                               inplace=True)
+        return (dxq, dxk, dv, _wgrad(dqw, q_w), _wgrad(dkw, k_w), None, None, None, None, None, None, None, None,
+                None)
+
+
+def packed_doc_attention(xq, xk, xv, q_norm_w=None, k_norm_w=None, rope_cos=None, rope_sin=None, position_ids=None,
+                         document_ids=None, scale=None, causal=True, sliding_window=None, eps=1e-6, tile_map=None):
+    """Keyword-friendly wrapper of ``PackedDocAttention.apply``; ``scale`` defaults to ``D**-0.5``."""
+    if scale is None:
+        scale = xq.shape[-1] ** -0.5
+    return PackedDocAttention.apply(xq, xk, xv, q_norm_w, k_norm_w, rope_cos, rope_sin, position_ids, document_ids,
+                                    float(scale), bool(causal), sliding_window, float(eps), tile_map)
+
+
+def qk_norm_rope(xq, xk, q_norm_w, k_norm_w, rope_cos, rope_sin, position_ids=None, eps=1e-6, add_unit_offset=True):
+    """The prologue on its own (differentiable): returns (q, k) in [B,S,H,D]."""
+    return _QKNormRope.apply(xq, xk, q_norm_w, k_norm_w, rope_cos, rope_sin, position_ids, float(eps),
+                             bool(add_unit_offset))
+
+
+def doc_masked_attention(q, k, v, document_ids=None, scale=None, causal=True, sliding_window=None, tile_map=None):
+    """The attention on its own (differentiable): q [B,S,Hq,D], k/v [B,S,Hkv,D] -> [B,S,Hq,D]."""
+    if scale is None:
+        scale = q.shape[-1] ** -0.5
+    return _DocMaskedAttention.apply(q, k, v, document_ids, float(scale), bool(causal), sliding_window, tile_map)

@@ -1,0 +1,234 @@
+// C-ABI layer: argument validation (runs on the host before any launch, so every error path is
+// reachable without a GPU) and dispatch to the kernel launchers.  See include/maester_attn.h.
+#include "common.h"
+
+#include <string.h>
+
+namespace ma {
+
+static thread_local char g_err[512] = "";
+
+void set_error(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+static int check_dims(const char* who, int B, int S, int Hq, int Hkv, int D) {
+    if (B <= 0 || S <= 0) return fail(MA_ERR_BAD_ARG, "%s: B=%d and S=%d must be positive", who, B, S);
+    if (Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0)
+        return fail(MA_ERR_BAD_ARG, "%s: Hq=%d must be a positive multiple of Hkv=%d", who, Hq, Hkv);
+    if (B > 65535 || Hq > 65535) return fail(MA_ERR_BAD_ARG, "%s: B=%d / Hq=%d exceed the grid limit 65535", who, B, Hq);
+    if ((int64_t)B * S > (int64_t)1 << 30) return fail(MA_ERR_BAD_ARG, "%s: B*S=%lld too large", who, (long long)B * S);
+    if (D != 64 && D != 128 && D != 256) return fail(MA_ERR_UNSUPPORTED, "%s: head_dim %d not in {64,128,256}", who, D);
+    return MA_OK;
+}
+
+static int check_dtype(const char* who, int dtype) {
+    if (dtype != MA_DTYPE_F32 && dtype != MA_DTYPE_BF16)
+        return fail(MA_ERR_BAD_ARG, "%s: dtype %d is neither MA_DTYPE_F32 nor MA_DTYPE_BF16", who, dtype);
+    return MA_OK;
+}
+
+static int check_tensor(const char* who, const char* name, const ma_tensor4* t, int dtype) {
+    if (!t || !t->ptr) return fail(MA_ERR_BAD_ARG, "%s: tensor %s is NULL", who, name);
+    const int elt = dtype == MA_DTYPE_BF16 ? 2 : 4;
+    // rows are moved with 16-byte vector accesses
+    const int64_t al = 16 / elt;
+    if (((uintptr_t)t->ptr & 15) != 0) return fail(MA_ERR_BAD_ARG, "%s: %s is not 16-byte aligned", who, name);
+    if (t->stride_b % al || t->stride_s % al || t->stride_h % al)
+        return fail(MA_ERR_BAD_ARG, "%s: strides of %s (%lld,%lld,%lld) must be multiples of %lld elements", who, name,
+                    (long long)t->stride_b, (long long)t->stride_s, (long long)t->stride_h, (long long)al);
+    if (t->stride_b < 0 || t->stride_s <= 0 || t->stride_h < 0)
+        return fail(MA_ERR_BAD_ARG, "%s: strides of %s must be non-negative (stride_s positive)", who, name);
+    return MA_OK;
+}
+
+static int check_map(const char* who, const ma_tile_map* m, bool need_kv, bool need_q) {
+    if (!m) return fail(MA_ERR_BAD_ARG, "%s: tile map is NULL", who);
+    if (need_kv && (!m->kv_num_blocks || !m->kv_indices || !m->full_kv_num_blocks || !m->full_kv_indices))
+        return fail(MA_ERR_BAD_ARG, "%s: tile map lacks the kv-side lists", who);
+    if (need_q && (!m->q_num_blocks || !m->q_indices || !m->full_q_num_blocks || !m->full_q_indices))
+        return fail(MA_ERR_BAD_ARG, "%s: tile map lacks the q-side lists", who);
+    return MA_OK;
+}
+
+static int check_mask(const char* who, int causal, int64_t window) {
+    if (causal != 0 && causal != 1) return fail(MA_ERR_BAD_ARG, "%s: causal must be 0 or 1, got %d", who, causal);
+    if (window < -1) return fail(MA_ERR_BAD_ARG, "%s: window must be -1 (none) or >= 0, got %lld", who, (long long)window);
+    return MA_OK;
+}
+
+}  // namespace ma
+
+using namespace ma;
+
+#define MA_TRY(expr)            \
+    do {                        \
+        int rc__ = (expr);      \
+        if (rc__) return rc__;  \
+    } while (0)
+
+extern "C" {
+
+int ma_version(void) { return 100; }
+
+const char* ma_last_error(void) { return g_err; }
+
+size_t ma_tile_map_workspace_bytes(int B, int S) {
+    if (B <= 0 || S <= 0) return 0;
+    const size_t T = ((size_t)S + MA_TILE - 1) / MA_TILE;
+    return (size_t)B * T * T;  // one class byte per tile
+}
+
+int ma_tile_map_build(const int64_t* document_ids, int B, int S, int causal, int64_t window, const ma_tile_map* out,
+                      void* workspace, size_t workspace_bytes, void* stream) {
+    const char* who = "ma_tile_map_build";
+    if (B <= 0 || S <= 0) return fail(MA_ERR_BAD_ARG, "%s: B=%d and S=%d must be positive", who, B, S);
+    if (B > 65535) return fail(MA_ERR_BAD_ARG, "%s: B=%d exceeds the grid limit 65535", who, B);
+    const int64_t T = ((int64_t)S + MA_TILE - 1) / MA_TILE;
+    if (T > 65535) return fail(MA_ERR_BAD_ARG, "%s: S=%d gives %lld tiles per side, limit 65535", who, S, (long long)T);
+    MA_TRY(check_mask(who, causal, window));
+    MA_TRY(check_map(who, out, true, true));
+    if (!workspace || workspace_bytes < ma_tile_map_workspace_bytes(B, S))
+        return fail(MA_ERR_BAD_ARG, "%s: workspace of %zu bytes, need %zu", who, workspace ? workspace_bytes : (size_t)0,
+                    ma_tile_map_workspace_bytes(B, S));
+    return launch_tile_map(document_ids, B, S, causal, window, *out, workspace, (hipStream_t)stream);
+}
+
+int ma_prologue_fwd(const ma_tensor4* q_in, const ma_tensor4* k_in, const ma_tensor4* q_out, const ma_tensor4* k_out,
+                    const float* q_weight, const float* k_weight, const float* rope_cos, const float* rope_sin,
+                    int64_t n_pos, const int64_t* position_ids, float eps, int add_unit_offset, float* q_rstd,
+                    float* k_rstd, int dtype, int B, int S, int Hq, int Hkv, int D, void* stream) {
+    const char* who = "ma_prologue_fwd";
+    MA_TRY(check_dims(who, B, S, Hq, Hkv, D));
+    MA_TRY(check_dtype(who, dtype));
+    MA_TRY(check_tensor(who, "q_in", q_in, dtype));
+    MA_TRY(check_tensor(who, "k_in", k_in, dtype));
+    MA_TRY(check_tensor(who, "q_out", q_out, dtype));
+    MA_TRY(check_tensor(who, "k_out", k_out, dtype));
+    if (!rope_cos || !rope_sin) return fail(MA_ERR_BAD_ARG, "%s: rope tables are NULL", who);
+    if (n_pos <= 0) return fail(MA_ERR_BAD_ARG, "%s: n_pos=%lld must be positive", who, (long long)n_pos);
+    if (!position_ids && n_pos < S)
+        return fail(MA_ERR_BAD_ARG, "%s: default positions need n_pos >= S (%lld < %d)", who, (long long)n_pos, S);
+    if (q_weight && !q_rstd) return fail(MA_ERR_BAD_ARG, "%s: q_rstd is NULL but q_weight is given", who);
+    if (k_weight && !k_rstd) return fail(MA_ERR_BAD_ARG, "%s: k_rstd is NULL but k_weight is given", who);
+    if (!(eps >= 0.f)) return fail(MA_ERR_BAD_ARG, "%s: eps must be >= 0", who);
+    return launch_prologue_fwd(*q_in, *k_in, *q_out, *k_out, q_weight, k_weight, rope_cos, rope_sin, n_pos,
+                               position_ids, eps, add_unit_offset ? 1 : 0, q_rstd, k_rstd, dtype, B, S, Hq, Hkv, D,
+                               (hipStream_t)stream);
+}
+
+size_t ma_prologue_bwd_workspace_bytes(int B, int S, int Hq, int Hkv, int D) {
+    (void)Hq; (void)Hkv;
+    if (B <= 0 || S <= 0 || D <= 0) return 0;
+    return (size_t)prologue_bwd_blocks(B, S) * 2 * (size_t)D * sizeof(float);
+}
+
+int ma_prologue_bwd(const ma_tensor4* q_in, const ma_tensor4* k_in, const ma_tensor4* dq_out, const ma_tensor4* dk_out,
+                    const ma_tensor4* dq_in, const ma_tensor4* dk_in, const float* q_weight, const float* k_weight,
+                    const float* rope_cos, const float* rope_sin, int64_t n_pos, const int64_t* position_ids,
+                    int add_unit_offset, const float* q_rstd, const float* k_rstd, float* dq_weight, float* dk_weight,
+                    void* workspace, size_t workspace_bytes, int dtype, int B, int S, int Hq, int Hkv, int D,
+                    void* stream) {
+    const char* who = "ma_prologue_bwd";
+    MA_TRY(check_dims(who, B, S, Hq, Hkv, D));
+    MA_TRY(check_dtype(who, dtype));
+    MA_TRY(check_tensor(who, "dq_out", dq_out, dtype));
+    MA_TRY(check_tensor(who, "dk_out", dk_out, dtype));
+    MA_TRY(check_tensor(who, "dq_in", dq_in, dtype));
+    MA_TRY(check_tensor(who, "dk_in", dk_in, dtype));
+    if (q_weight) MA_TRY(check_tensor(who, "q_in", q_in, dtype));
+    if (k_weight) MA_TRY(check_tensor(who, "k_in", k_in, dtype));
+    if (!rope_cos || !rope_sin) return fail(MA_ERR_BAD_ARG, "%s: rope tables are NULL", who);
+    if (n_pos <= 0) return fail(MA_ERR_BAD_ARG, "%s: n_pos=%lld must be positive", who, (long long)n_pos);
+    if (!position_ids && n_pos < S)
+        return fail(MA_ERR_BAD_ARG, "%s: default positions need n_pos >= S (%lld < %d)", who, (long long)n_pos, S);
+    if (q_weight && (!q_rstd || !dq_weight)) return fail(MA_ERR_BAD_ARG, "%s: q_weight needs q_rstd and dq_weight", who);
+    if (k_weight && (!k_rstd || !dk_weight)) return fail(MA_ERR_BAD_ARG, "%s: k_weight needs k_rstd and dk_weight", who);
+    if ((q_weight || k_weight) &&
+        (!workspace || workspace_bytes < ma_prologue_bwd_workspace_bytes(B, S, Hq, Hkv, D)))
+        return fail(MA_ERR_BAD_ARG, "%s: workspace of %zu bytes, need %zu", who, workspace ? workspace_bytes : (size_t)0,
+                    ma_prologue_bwd_workspace_bytes(B, S, Hq, Hkv, D));
+    ma_tensor4 none = {nullptr, 0, 0, 0};
+    return launch_prologue_bwd(q_in ? *q_in : none, k_in ? *k_in : none, *dq_out, *dk_out, *dq_in, *dk_in, q_weight,
+                               k_weight, rope_cos, rope_sin, n_pos, position_ids, add_unit_offset ? 1 : 0, q_rstd,
+                               k_rstd, dq_weight, dk_weight, workspace, dtype, B, S, Hq, Hkv, D, (hipStream_t)stream);
+}
+
+static int fill_attn(const char* who, AttnArgs& a, const ma_tensor4* q, const ma_tensor4* k, const ma_tensor4* v,
+                     const ma_tensor4* out, const ma_tile_map* map, const int64_t* document_ids, int causal,
+                     int64_t window, float scale, int dtype, int B, int S, int Hq, int Hkv, int D, bool bwd) {
+    MA_TRY(check_dims(who, B, S, Hq, Hkv, D));
+    MA_TRY(check_dtype(who, dtype));
+    MA_TRY(check_tensor(who, "q", q, dtype));
+    MA_TRY(check_tensor(who, "k", k, dtype));
+    MA_TRY(check_tensor(who, "v", v, dtype));
+    MA_TRY(check_tensor(who, "out", out, dtype));
+    MA_TRY(check_mask(who, causal, window));
+    MA_TRY(check_map(who, map, true, bwd));
+    if (!(scale > 0.f) || scale != scale) return fail(MA_ERR_BAD_ARG, "%s: scale must be positive and finite", who);
+    memset(&a, 0, sizeof(a));
+    a.q = *q; a.k = *k; a.v = *v; a.o = *out;
+    a.map = *map;
+    a.doc = document_ids;
+    a.causal = causal;
+    a.window = window;
+    a.scale = scale;
+    a.B = B; a.S = S; a.Hq = Hq; a.Hkv = Hkv; a.D = D;
+    a.T = (S + MA_TILE - 1) / MA_TILE;
+    return MA_OK;
+}
+
+int ma_attn_fwd(const ma_tensor4* q, const ma_tensor4* k, const ma_tensor4* v, const ma_tensor4* out, float* lse,
+                const ma_tile_map* map, const int64_t* document_ids, int causal, int64_t window, float scale, int dtype,
+                int B, int S, int Hq, int Hkv, int D, void* stream) {
+    const char* who = "ma_attn_fwd";
+    AttnArgs a;
+    MA_TRY(fill_attn(who, a, q, k, v, out, map, document_ids, causal, window, scale, dtype, B, S, Hq, Hkv, D, false));
+    if (!lse) return fail(MA_ERR_BAD_ARG, "%s: lse is NULL", who);
+    a.lse = lse;
+    return dtype == MA_DTYPE_BF16 ? launch_attn_fwd_bf16(a, (hipStream_t)stream)
+                                  : launch_attn_fwd_f32(a, (hipStream_t)stream);
+}
+
+size_t ma_attn_bwd_workspace_bytes(int B, int S, int Hq, int Hkv, int D) {
+    (void)Hkv; (void)D;
+    if (B <= 0 || S <= 0 || Hq <= 0) return 0;
+    return (size_t)B * Hq * S * sizeof(float);  // delta
+}
+
+int ma_attn_bwd(const ma_tensor4* q, const ma_tensor4* k, const ma_tensor4* v, const ma_tensor4* out,
+                const ma_tensor4* dout, const float* lse, const ma_tensor4* dq, const ma_tensor4* dk,
+                const ma_tensor4* dv, const ma_tile_map* map, const int64_t* document_ids, int causal, int64_t window,
+                float scale, void* workspace, size_t workspace_bytes, int dtype, int B, int S, int Hq, int Hkv, int D,
+                void* stream) {
+    const char* who = "ma_attn_bwd";
+    AttnArgs a;
+    MA_TRY(fill_attn(who, a, q, k, v, out, map, document_ids, causal, window, scale, dtype, B, S, Hq, Hkv, D, true));
+    MA_TRY(check_tensor(who, "dout", dout, dtype));
+    MA_TRY(check_tensor(who, "dq", dq, dtype));
+    MA_TRY(check_tensor(who, "dk", dk, dtype));
+    MA_TRY(check_tensor(who, "dv", dv, dtype));
+    if (!lse) return fail(MA_ERR_BAD_ARG, "%s: lse is NULL", who);
+    if (!workspace || workspace_bytes < ma_attn_bwd_workspace_bytes(B, S, Hq, Hkv, D))
+        return fail(MA_ERR_BAD_ARG, "%s: workspace of %zu bytes, need %zu", who, workspace ? workspace_bytes : (size_t)0,
+                    ma_attn_bwd_workspace_bytes(B, S, Hq, Hkv, D));
+    if (((uintptr_t)workspace & 15) != 0) return fail(MA_ERR_BAD_ARG, "%s: workspace is not 16-byte aligned", who);
+    a.dout = *dout; a.dq = *dq; a.dk = *dk; a.dv = *dv;
+    a.lse = (float*)lse;
+    a.delta = (float*)workspace;
+    return dtype == MA_DTYPE_BF16 ? launch_attn_bwd_bf16(a, (hipStream_t)stream)
+                                  : launch_attn_bwd_f32(a, (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,103 @@
+// Block-sparse tile map from document_ids, in torch's BlockMask format.
+//
+// Stands in for create_block_mask(make_document_mask_wrapper(...), B, None, S, S)
+// (maester/models/gemma/model.py:694-730), which materialises a [B,1,S,S] bool and block-reduces
+// it (torch/nn/attention/flex_attention.py:979-1022, 429-441).  Here every 128x128 tile is
+// classified directly from the two 128-id slices it covers (exact for arbitrary ids, no S^2
+// memory), then the ordered lists are emitted: set tiles ascending, unset tiles ascending.
+#include "common.h"
+
+namespace ma {
+
+// class codes in the workspace: 0 empty, 1 partial, 2 full
+__global__ __launch_bounds__(kTile) void classify_tiles_kernel(const int64_t* __restrict__ doc, int S, int T,
+                                                                int causal, int64_t window,
+                                                                uint8_t* __restrict__ cls) {
+    const int j = blockIdx.x, i = blockIdx.y, b = blockIdx.z;
+    uint8_t* out = cls + ((size_t)b * T + i) * T + j;
+    const int q0 = i * kTile, k0 = j * kTile;
+    // tiles the base predicate rules out entirely (uniform over the workgroup)
+    bool dead = false;
+    if ((causal || window >= 0) && k0 > q0 + kTile - 1) dead = true;
+    if (window >= 0 && (int64_t)q0 - (int64_t)(k0 + kTile - 1) > window) dead = true;
+    if (dead) {
+        if (threadIdx.x == 0) *out = 0;
+        return;
+    }
+    __shared__ int64_t kdoc[kTile];
+    __shared__ int wave_cnt[kTile / 64];
+    const int t = threadIdx.x;
+    const int64_t* drow = doc ? doc + (size_t)b * S : nullptr;
+    if (drow) kdoc[t] = (k0 + t < S) ? drow[k0 + t] : 0;
+    __syncthreads();
+    const int q = q0 + t;
+    int cnt = 0;
+    if (q < S) {
+        const int64_t dq = drow ? drow[q] : 0;
+        const int kmax = min(kTile, S - k0);
+        for (int c = 0; c < kmax; ++c) {
+            bool ok = pair_allowed(q, k0 + c, causal, window);
+            if (drow) ok = ok && (kdoc[c] == dq);
+            cnt += ok ? 1 : 0;
+        }
+    }
+    for (int off = 32; off > 0; off >>= 1) cnt += __shfl_down(cnt, off, 64);
+    if ((t & 63) == 0) wave_cnt[t >> 6] = cnt;
+    __syncthreads();
+    if (t == 0) {
+        int total = 0;
+        for (int w = 0; w < kTile / 64; ++w) total += wave_cnt[w];
+        *out = total == 0 ? 0 : (total == kTile * kTile ? 2 : 1);
+    }
+}
+
+// One wave per (list kind, batch row, tile row).  kind: 0 kv partial, 1 kv full, 2 q partial, 3 q full.
+__global__ __launch_bounds__(64) void order_lists_kernel(const uint8_t* __restrict__ cls, int T, ma_tile_map out) {
+    const int r = blockIdx.x, b = blockIdx.y, kind = blockIdx.z;
+    const int lane = threadIdx.x;
+    const uint8_t want = (kind & 1) ? 2 : 1;
+    const bool transposed = kind >= 2;
+    const uint8_t* base = cls + (size_t)b * T * T;
+    int32_t* num = kind == 0 ? out.kv_num_blocks : kind == 1 ? out.full_kv_num_blocks
+                 : kind == 2 ? out.q_num_blocks : out.full_q_num_blocks;
+    int32_t* idx = kind == 0 ? out.kv_indices : kind == 1 ? out.full_kv_indices
+                 : kind == 2 ? out.q_indices : out.full_q_indices;
+    num += (size_t)b * T + r;
+    idx += ((size_t)b * T + r) * T;
+
+    int total = 0;
+    for (int c0 = 0; c0 < T; c0 += 64) {
+        const int c = c0 + lane;
+        bool set = false;
+        if (c < T) set = (transposed ? base[(size_t)c * T + r] : base[(size_t)r * T + c]) == want;
+        total += __popcll(__ballot(set));
+    }
+    int seen_set = 0;
+    for (int c0 = 0; c0 < T; c0 += 64) {
+        const int c = c0 + lane;
+        bool set = false;
+        if (c < T) set = (transposed ? base[(size_t)c * T + r] : base[(size_t)r * T + c]) == want;
+        const unsigned long long m = __ballot(set);
+        const int before = __popcll(m & ((1ull << lane) - 1ull));
+        if (c < T) {
+            const int set_before = seen_set + before;
+            const int pos = set ? set_before : total + (c - set_before);
+            idx[pos] = c;
+        }
+        seen_set += __popcll(m);
+    }
+    if (lane == 0) *num = total;
+}
+
+int launch_tile_map(const int64_t* doc, int B, int S, int causal, int64_t window, const ma_tile_map& out,
+                    void* ws, hipStream_t st) {
+    const int T = (S + kTile - 1) / kTile;
+    uint8_t* cls = (uint8_t*)ws;
+    hipLaunchKernelGGL(classify_tiles_kernel, dim3(T, T, B), dim3(kTile), 0, st, doc, S, T, causal, window, cls);
+    int rc = check_launch("classify_tiles_kernel");
+    if (rc) return rc;
+    hipLaunchKernelGGL(order_lists_kernel, dim3(T, B, 4), dim3(64), 0, st, cls, T, out);
+    return check_launch("order_lists_kernel");
+}
+
+}  // namespace ma

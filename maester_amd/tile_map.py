@@ -1,0 +1,85 @@
+"""Block-sparse tile map (torch ``BlockMask`` format) built on the GPU from ``document_ids``.
+
+Replaces the two per-step ``create_block_mask(make_document_mask_wrapper(...), B, None, S, S)``
+calls of maester/models/gemma/model.py:694-730.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from ctypes import byref, c_void_p
+
+import torch
+
+from . import _lib
+
+TILE = _lib.MA_TILE
+
+
+@dataclass
+class TileMap:
+    """The eight ``BlockMask`` tensors (head dim 1) plus the mask parameters they were built for.
+
+    Field names, shapes ([B,1,T] / [B,1,T,T]) and dtype (int32) are those of
+    ``torch.nn.attention.flex_attention.BlockMask``; ``BLOCK_SIZE`` is (128, 128)."""
+    kv_num_blocks: torch.Tensor
+    kv_indices: torch.Tensor
+    full_kv_num_blocks: torch.Tensor
+    full_kv_indices: torch.Tensor
+    q_num_blocks: torch.Tensor
+    q_indices: torch.Tensor
+    full_q_num_blocks: torch.Tensor
+    full_q_indices: torch.Tensor
+    seq_len: int
+    causal: bool
+    window: int | None
+    BLOCK_SIZE: tuple = (TILE, TILE)
+
+    NAMES = ("kv_num_blocks", "kv_indices", "full_kv_num_blocks", "full_kv_indices",
+             "q_num_blocks", "q_indices", "full_q_num_blocks", "full_q_indices")
+
+    def as_dict(self) -> dict:
+        return {n: getattr(self, n) for n in self.NAMES}
+
+    def c_struct(self) -> _lib.MaTileMap:
+        return _lib.MaTileMap(*[c_void_p(getattr(self, n).data_ptr()) for n in self.NAMES])
+
+    @property
+    def seq_lengths(self):
+        return (self.seq_len, self.seq_len)
+
+    def sparsity(self) -> float:
+        """Fraction of tiles never visited (the skipped-tile ratio)."""
+        B, _, T = self.kv_num_blocks.shape
+        visited = int(self.kv_num_blocks.sum()) + int(self.full_kv_num_blocks.sum())
+        return 1.0 - visited / float(B * T * T)
+
+
+def build_tile_map(document_ids: torch.Tensor | None, batch_size: int, seq_len: int, causal: bool = True,
+                   sliding_window: int | None = None, device=None) -> TileMap:
+    """``document_ids``: int64 [B,S] on the GPU, or ``None`` for the plain causal / sliding-window
+    mask (maester/models/gemma/model.py:227-228).  ``sliding_window`` is inclusive (``q - kv <= W``,
+    model.py:206-207) and implies causality."""
+    if document_ids is not None:
+        _lib.require_gpu(document_ids, "build_tile_map")
+        if document_ids.shape != (batch_size, seq_len):
+            raise ValueError(f"document_ids shape {tuple(document_ids.shape)} != {(batch_size, seq_len)}")
+        document_ids = document_ids.detach().to(torch.long).contiguous()
+        device = document_ids.device
+    elif device is None:
+        device = torch.device("cuda", torch.cuda.current_device())
+    device = torch.device(device)
+    L = _lib.lib()
+    T = (seq_len + TILE - 1) // TILE
+    nums = torch.empty(4, batch_size, 1, T, dtype=torch.int32, device=device)
+    idxs = torch.empty(4, batch_size, 1, T, T, dtype=torch.int32, device=device)
+    tm = TileMap(nums[0], idxs[0], nums[1], idxs[1], nums[2], idxs[2], nums[3], idxs[3],
+                 seq_len=seq_len, causal=bool(causal), window=sliding_window)
+    ws_bytes = L.ma_tile_map_workspace_bytes(batch_size, seq_len)
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=device)
+    cs = tm.c_struct()
+    with torch.cuda.device(device):
+        rc = L.ma_tile_map_build(_lib.ptr(document_ids), batch_size, seq_len, 1 if causal else 0,
+                                 -1 if sliding_window is None else int(sliding_window), byref(cs),
+                                 _lib.ptr(ws), ws_bytes, _lib.current_stream(device))
+    _lib.check(rc)
+    return tm

@@ -1,0 +1,197 @@
+"""HIP attention (through the C ABI) vs the oracle.
+
+Tolerances (the stated bar of the path): fp32 activations <= 1e-4 max-abs; bf16 activations
+<= 2e-2 max-abs and <= 1e-2 relative L2 against the oracle evaluated in fp32 on the same
+(bf16-rounded) inputs."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import max_abs, rel_l2
+from maester_amd import build_tile_map, doc_masked_attention, packed_doc_attention, workloads
+from maester_amd.attention import attention_forward
+from oracle import attention as A
+from oracle import prologue as P
+
+pytestmark = pytest.mark.gpu
+
+BF16_MAX_ABS, BF16_REL_L2, FP32_MAX_ABS = 2e-2, 1e-2, 1e-4
+
+
+def _ids(B, S, seed, kind="docs"):
+    rng = np.random.default_rng(seed)
+    if kind == "none":
+        return None
+    ids = np.zeros((B, S), dtype=np.int64)
+    for b in range(B):
+        cuts = np.sort(rng.integers(1, S, size=max(1, S // 150)))
+        for c in cuts:
+            ids[b, c:] += 1
+    if kind == "padded":
+        ids[:, S - S // 7:] = -1
+    return torch.from_numpy(ids)
+
+
+def _qkv(B, S, Hq, Hkv, D, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    mk = lambda h: torch.randn(B, S, h, D, generator=g).to(dtype)
+    return mk(Hq), mk(Hkv), mk(Hkv), mk(Hq)
+
+
+def _check(got, want, dtype, tag):
+    if dtype == torch.float32:
+        assert max_abs(got.cpu(), want) <= FP32_MAX_ABS, (tag, max_abs(got.cpu(), want))
+    else:
+        ma, rl = max_abs(got.cpu(), want), rel_l2(got.cpu(), want)
+        scale = max(1.0, float(want.abs().max()))
+        assert ma <= BF16_MAX_ABS * scale and rl <= BF16_REL_L2, (tag, ma, rl, scale)
+
+
+# ------------------------------------------------------------------ fp32 path ------------------
+def test_c1_full_config_fp32(gpu):
+    """Config 1 end to end (prologue + attention), fp32, forward only, <= 1e-4 max-abs."""
+    wl = workloads.make("c1")
+    want = A.full_path(wl.xq, wl.xk, wl.xv, wl.q_w, wl.k_w, wl.cos, wl.sin, wl.position_ids, wl.document_ids, wl.scale,
+                       compute_dtype=torch.float64)
+    g = wl.to(gpu)
+    out = packed_doc_attention(g.xq, g.xk, g.xv, g.q_w, g.k_w, g.cos, g.sin, g.position_ids, g.document_ids, g.scale)
+    assert out.dtype == torch.float32 and out.shape == wl.xq.shape
+    assert max_abs(out.cpu(), want) <= FP32_MAX_ABS
+    # and against torch's own FlexAttention on the CPU, fed the oracle prologue
+    q, k = P.prologue(wl.xq, wl.xk, wl.q_w, wl.k_w, wl.cos, wl.sin, wl.position_ids)
+    flex = A.flex_attention_cpu(q, k, wl.xv, wl.document_ids, wl.scale)
+    assert max_abs(out.cpu(), flex) <= FP32_MAX_ABS
+
+
+def test_reference_known_answers_fp32(gpu):
+    # maester tests/test_packed_sft.py:164-212 -- boundary inside a 128-block, exact -1 / +1
+    S, D, boundary = 256, 64, 176
+    ids = torch.zeros((1, S), dtype=torch.long); ids[:, boundary:] = 1
+    q = torch.ones(1, S, 1, D); k = torch.ones_like(q); v = torch.ones_like(q); v[:, :boundary] = -1
+    out = doc_masked_attention(q.to(gpu), k.to(gpu), v.to(gpu), ids.to(gpu), D ** -0.5).cpu()[0, :, 0]
+    assert torch.allclose(out[:boundary], torch.full_like(out[:boundary], -1))
+    assert torch.allclose(out[boundary:], torch.ones_like(out[boundary:]))
+    # tests/test_packed_sft.py:104-162 -- 4 docs of 32 in one block, vs dense softmax atol 1e-5 rtol 1e-4
+    torch.manual_seed(0)
+    ids = torch.zeros((1, 128), dtype=torch.long); ids[:, 32:64] = 1; ids[:, 64:96] = 2; ids[:, 96:] = 3
+    q, k, v = (torch.randn(1, 128, 2, 64) for _ in range(3))
+    got = doc_masked_attention(q.to(gpu), k.to(gpu), v.to(gpu), ids.to(gpu), 64 ** -0.5).cpu()
+    assert torch.allclose(got, A.dense_attention(q, k, v, ids, 64 ** -0.5), atol=1e-5, rtol=1e-4)
+
+
+@pytest.mark.parametrize("D,S,window,kind", [(64, 300, None, "docs"), (128, 513, 100, "padded"), (64, 256, 0, "none"),
+                                             (256, 200, None, "docs")])
+def test_fp32_forward_edge_cases(gpu, D, S, window, kind):
+    B, Hq, Hkv = 2, 4, 2
+    q, k, v, _ = _qkv(B, S, Hq, Hkv, D, torch.float32, 1)
+    ids = _ids(B, S, 2, kind)
+    want, wl = A.dense_attention(q, k, v, ids, 0.2, True, window, compute_dtype=torch.float64, return_lse=True)
+    tm = build_tile_map(None if ids is None else ids.to(gpu), B, S, True, window, device=gpu)
+    out, lse = attention_forward(q.to(gpu), k.to(gpu), v.to(gpu), tm, None if ids is None else ids.to(gpu), 0.2, True, window)
+    assert max_abs(out.cpu(), want) <= FP32_MAX_ABS and max_abs(lse.cpu(), wl) <= FP32_MAX_ABS
+
+
+@pytest.mark.parametrize("D", [64, 128])
+def test_fp32_backward(gpu, D):
+    B, S, Hq, Hkv = 1, 400, 4, 2
+    q, k, v, do = _qkv(B, S, Hq, Hkv, D, torch.float32, 3)
+    ids = _ids(B, S, 4)
+    _, dq, dk, dv = A.dense_attention_fwd_bwd(q, k, v, do, ids, 0.15, True, 150, compute_dtype=torch.float64)
+    hq, hk, hv = (t.to(gpu).requires_grad_() for t in (q, k, v))
+    out = doc_masked_attention(hq, hk, hv, ids.to(gpu), 0.15, True, 150)
+    gq, gk, gv = torch.autograd.grad(out, (hq, hk, hv), do.to(gpu))
+    for a, b in ((gq, dq), (gk, dk), (gv, dv)):
+        assert max_abs(a.cpu(), b) <= FP32_MAX_ABS
+
+
+# ------------------------------------------------------------------ bf16 MFMA path -------------
+BF16_CASES = [
+    # name, B, S, Hq, Hkv, D, window, ids kind
+    ("gemma4b_global_small", 2, 1024, 4, 2, 256, None, "docs"),
+    ("gemma4b_local_small", 2, 1024, 4, 2, 256, 300, "docs"),
+    ("llama_shape_small", 1, 1024, 8, 2, 128, None, "docs"),
+    ("ragged_padded", 2, 777, 2, 1, 256, None, "padded"),
+    ("ragged_window_d128", 1, 333, 4, 4, 128, 64, "docs"),
+    ("no_ids_causal", 1, 640, 2, 1, 256, None, "none"),
+    ("d64", 1, 512, 2, 2, 64, None, "docs"),
+    ("tiny_one_tile", 1, 50, 2, 1, 128, None, "docs"),
+]
+
+
+@pytest.mark.parametrize("case", BF16_CASES, ids=[c[0] for c in BF16_CASES])
+def test_bf16_forward(gpu, case):
+    _, B, S, Hq, Hkv, D, window, kind = case
+    q, k, v, _ = _qkv(B, S, Hq, Hkv, D, torch.bfloat16, 5)
+    ids = _ids(B, S, 6, kind)
+    scale = D ** -0.5
+    want, wl = A.dense_attention(q, k, v, ids, scale, True, window, return_lse=True)
+    gids = None if ids is None else ids.to(gpu)
+    tm = build_tile_map(gids, B, S, True, window, device=gpu)
+    out, lse = attention_forward(q.to(gpu), k.to(gpu), v.to(gpu), tm, gids, scale, True, window)
+    assert out.dtype == torch.bfloat16
+    _check(out, want, torch.bfloat16, case[0])
+    assert max_abs(lse.cpu(), wl) <= 2e-2
+
+
+@pytest.mark.parametrize("case", BF16_CASES, ids=[c[0] for c in BF16_CASES])
+def test_bf16_backward(gpu, case):
+    _, B, S, Hq, Hkv, D, window, kind = case
+    q, k, v, do = _qkv(B, S, Hq, Hkv, D, torch.bfloat16, 7)
+    ids = _ids(B, S, 8, kind)
+    scale = D ** -0.5
+    _, dq, dk, dv = A.dense_attention_fwd_bwd(q, k, v, do, ids, scale, True, window)
+    gids = None if ids is None else ids.to(gpu)
+    hq, hk, hv = (t.to(gpu).requires_grad_() for t in (q, k, v))
+    out = doc_masked_attention(hq, hk, hv, gids, scale, True, window)
+    gq, gk, gv = torch.autograd.grad(out, (hq, hk, hv), do.to(gpu))
+    for name, a, b in (("dq", gq, dq), ("dk", gk, dk), ("dv", gv, dv)):
+        _check(a, b, torch.bfloat16, (case[0], name))
+    # dK/dV/dQ are produced without atomics: a second run is bit-identical
+    out2 = doc_masked_attention(hq, hk, hv, gids, scale, True, window)
+    g2 = torch.autograd.grad(out2, (hq, hk, hv), do.to(gpu))
+    assert all(torch.equal(x, y) for x, y in zip(g2, (gq, gk, gv)))
+
+
+def test_full_path_bf16_with_norm_weights(gpu):
+    """Prologue + attention + both backward stages through PackedDocAttention, incl. dW of the norms."""
+    wl = workloads.make("c2", B=1, S=1024)
+    ins = [wl.xq.float().requires_grad_(), wl.xk.float().requires_grad_(), wl.xv.float().requires_grad_(),
+           wl.q_w.clone().requires_grad_(), wl.k_w.clone().requires_grad_()]
+    ref = A.full_path(ins[0], ins[1], ins[2], ins[3], ins[4], wl.cos, wl.sin, wl.position_ids, wl.document_ids, wl.scale)
+    want = torch.autograd.grad(ref, ins, wl.dout.float())
+    g = wl.to(gpu)
+    hin = [g.xq.clone().requires_grad_(), g.xk.clone().requires_grad_(), g.xv.clone().requires_grad_(),
+           g.q_w.clone().requires_grad_(), g.k_w.clone().requires_grad_()]
+    out = packed_doc_attention(hin[0], hin[1], hin[2], hin[3], hin[4], g.cos, g.sin, g.position_ids, g.document_ids, g.scale)
+    _check(out, ref.detach(), torch.bfloat16, "out")
+    got = torch.autograd.grad(out, hin, g.dout)
+    for name, a, b in zip(("dxq", "dxk", "dxv", "dq_w", "dk_w"), got, want):
+        _check(a, b, torch.bfloat16, name)
+
+
+@pytest.mark.parametrize("name", ["c2", "c3", "c5"])
+def test_full_size_properties_and_slice(gpu, name):
+    """At the benchmark shapes: one (row, kv head) slice against the oracle evaluated on the GPU, plus
+    size-independent properties (constant V -> constant output, linearity in V, determinism)."""
+    wl = workloads.make(name).to(gpu)
+    sp = wl.spec
+    q, k = wl.xq, wl.xk                                   # attention only: feed raw activations
+    tm = build_tile_map(wl.document_ids, sp.B, sp.S, True, sp.window)
+    out, lse = attention_forward(q, k, wl.xv, tm, wl.document_ids, wl.scale, True, sp.window)
+    G = sp.Hq // sp.Hkv
+    b, hk = sp.B - 1, sp.Hkv - 1
+    want, wlse = A.dense_attention(q[b:b + 1, :, hk * G:(hk + 1) * G], k[b:b + 1, :, hk:hk + 1], wl.xv[b:b + 1, :, hk:hk + 1],
+                                   wl.document_ids[b:b + 1], wl.scale, True, sp.window, return_lse=True)
+    _check(out[b:b + 1, :, hk * G:(hk + 1) * G], want.cpu(), torch.bfloat16, name)
+    assert max_abs(lse[b:b + 1, hk * G:(hk + 1) * G].cpu(), wlse.cpu()) <= 2e-2
+    ones = torch.ones_like(wl.xv)
+    o1, _ = attention_forward(q, k, ones, tm, wl.document_ids, wl.scale, True, sp.window)
+    assert max_abs(o1.cpu(), torch.ones_like(o1).cpu()) <= 1e-2            # softmax rows sum to one
+    o2, _ = attention_forward(q, k, wl.xv * 2, tm, wl.document_ids, wl.scale, True, sp.window)
+    assert torch.equal(o2.float(), out.float() * 2)                        # exact: scaling V by 2 is exact in bf16
+    o3, l3 = attention_forward(q, k, wl.xv, tm, wl.document_ids, wl.scale, True, sp.window)
+    assert torch.equal(o3, out) and torch.equal(l3, lse)
+    # first token of every document attends only to itself
+    starts = (wl.position_ids == 0)
+    for h in (0, sp.Hq - 1):
+        assert torch.equal(out[:, :, h][starts], wl.xv[:, :, h // G][starts])

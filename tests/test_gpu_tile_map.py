@@ -1,0 +1,74 @@
+"""HIP tile map vs the oracle: bit-exact on all eight BlockMask tensors, tails included."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from maester_amd import build_tile_map, workloads
+from oracle import tile_map as otm
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "tile_lists.json")
+
+
+def _assert_equal(tm, want, tag):
+    got = tm.as_dict()
+    for k in otm.NAMES:
+        assert got[k].dtype == torch.int32 and got[k].is_contiguous()
+        assert got[k].shape == want[k].shape, (tag, k, got[k].shape, want[k].shape)
+        assert torch.equal(got[k].cpu(), want[k]), (tag, k)
+
+
+def test_golden_fixture_through_c_abi(gpu):
+    with open(GOLDEN) as f:
+        gold = json.load(f)
+    for case in gold["cases"]:
+        ids = None if case["document_ids"] is None else torch.tensor(case["document_ids"], dtype=torch.long, device=gpu)
+        tm = build_tile_map(ids, case["B"], case["S"], case["causal"], case["window"], device=gpu)
+        want = {k: torch.tensor(v, dtype=torch.int32) for k, v in case["expect"].items()}
+        _assert_equal(tm, want, case["name"])
+
+
+def test_against_torch_create_block_mask_small(gpu):
+    rng = np.random.default_rng(11)
+    for S in (128, 200, 256, 384, 512, 1000):
+        ids = torch.from_numpy(np.sort(rng.integers(0, 4, size=(2, S)), axis=1))
+        for causal, window in [(True, None), (True, 100), (True, 0), (False, None)]:
+            want = otm.block_mask_to_dict(otm.torch_block_mask(ids, 2, S, causal, window))
+            tm = build_tile_map(ids.to(gpu), 2, S, causal, window)
+            _assert_equal(tm, want, (S, causal, window))
+    # arbitrary (non-contiguous) ids and the no-ids masks
+    ids = torch.from_numpy(rng.integers(0, 3, size=(1, 700)))
+    _assert_equal(build_tile_map(ids.to(gpu), 1, 700), otm.tile_lists(ids, 1, 700), "random ids")
+    for window in (None, 300):
+        _assert_equal(build_tile_map(None, 3, 900, True, window, device=gpu), otm.tile_lists(None, 3, 900, True, window),
+                      ("no ids", window))
+
+
+@pytest.mark.parametrize("name", ["c1", "c2", "c3", "c4", "c5"])
+def test_full_size_configs(gpu, name):
+    sp = workloads.spec(name)
+    rows = workloads.document_lengths(sp)
+    _, doc = workloads.ids_from_lengths(rows, sp.S)
+    want = otm.tile_lists_c(doc, sp.B, sp.S, True, sp.window)
+    tm = build_tile_map(doc.to(gpu), sp.B, sp.S, True, sp.window)
+    _assert_equal(tm, want, name)
+    # the survey's tile census for these seeded layouts
+    census = {"c1": (35, 4), "c2": (684, 1014), "c3": (632, 752), "c4": (420, 8296), "c5": (602, 2437)}
+    assert (int(tm.kv_num_blocks.sum()), int(tm.full_kv_num_blocks.sum())) == census[name]
+    assert int(tm.q_num_blocks.sum()) == census[name][0] and int(tm.full_q_num_blocks.sum()) == census[name][1]
+
+
+def test_padding_tail_and_large_T(gpu):
+    sp = workloads.spec("c2")
+    rows = workloads.document_lengths(sp)
+    _, doc = workloads.ids_from_lengths(rows, sp.S, pad_tail=777)
+    assert (doc[:, -777:] == -1).all()
+    _assert_equal(build_tile_map(doc.to(gpu), sp.B, sp.S, True, 1024), otm.tile_lists_c(doc, sp.B, sp.S, True, 1024), "pad")
+    # more than 64 tiles per row exercises the multi-pass ordered-list kernel
+    S = 128 * 150 + 17
+    ids = torch.zeros((1, S), dtype=torch.long)
+    ids[:, 5000:12000] = 1; ids[:, 12000:] = 2
+    _assert_equal(build_tile_map(ids.to(gpu), 1, S, True, 4096), otm.tile_lists_c(ids, 1, S, True, 4096), "T=151")
