@@ -1,0 +1,232 @@
+#!/usr/bin/env python3
+"""Benchmark of the packed-SFT document-masked attention path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2] [--no-cpu-baseline]
+
+A step is one pass of the attention hot path over one batch of synthetic input already resident in
+HBM: ``ma_attn_fwd`` followed by ``ma_attn_bwd`` (delta, dK/dV, dQ kernels) through the C ABI.
+The headline value is useful TFLOP/s = 12*D*Hq*N_pairs / step time, N_pairs = unmasked (q, kv)
+pairs (the MFU convention of maester/models/gemma/model.py:71-75: 2 forward + 4 backward GEMMs,
+recompute not counted), for the Gemma-3-4B global-layer shape.  The same run also times, each in
+its own bracket: every kernel alone (HIP events on the launch stream), the fused QK-RMSNorm+RoPE
+prologue (HBM roofline), the tile-map build, the whole autograd Function, and a bounded CPU sample
+of the oracle on the host cores.  Prints ONE JSON line.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_DENSE_TFLOPS = 2500.0   # MI355X bf16 dense MFMA: 256 CU x 4096 FLOP/clk/CU x 2.4 GHz
+PEAK_HBM_GBPS = 8000.0            # MI355X HBM3E
+
+
+def _events(n):
+    return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
+
+
+def time_region(fn, steps, warmup):
+    """Average milliseconds per call, HIP events on the current (launch) stream."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    a, b = _events(2)
+    a.record()
+    for _ in range(steps):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / steps
+
+
+def cpu_baseline(wl, seconds_hint=20.0):
+    """The oracle (a CPU restatement: 'port') timed on the host cores on ONE (batch row, kv head)
+    slice of the same workload, forward + backward through torch autograd."""
+    from oracle import attention as OA
+    sp = wl.spec
+    G = sp.Hq // sp.Hkv
+    b, hk = 0, 0
+    q = wl.xq[b:b + 1, :, hk * G:(hk + 1) * G].float()
+    k = wl.xk[b:b + 1, :, hk:hk + 1].float()
+    v = wl.xv[b:b + 1, :, hk:hk + 1].float()
+    do = wl.dout[b:b + 1, :, hk * G:(hk + 1) * G].float()
+    ids = wl.document_ids[b:b + 1]
+    t0 = time.perf_counter()
+    OA.dense_attention_fwd_bwd(q, k, v, do, ids, wl.scale, True, sp.window)
+    dt = time.perf_counter() - t0
+    from maester_amd import workloads as W
+    pairs = W.count_pairs([wl.doc_lengths[b]], sp.window)
+    flops = 12 * sp.D * G * pairs
+    return {
+        "value": flops / dt / 1e12, "unit": "useful TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+        "sample": f"oracle dense fwd+bwd (fp32, torch CPU) on 1 of {sp.B * sp.Hkv} (batch row, kv head) slices "
+                  f"of {sp.name}: S={sp.S}, G={G}, D={sp.D}; {dt:.2f} s",
+        "seconds": dt,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="c2")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this path is measured on ONE GPU; --gpus N with N > 1 is not run "
+              "(the path shards over batch rows / kv heads with no exchange, see DESIGN.md).", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP path has no CPU fallback.", file=sys.stderr)
+        sys.exit(3)
+
+    from maester_amd import _lib, build_tile_map, packed_doc_attention, workloads
+    from maester_amd.attention import (attention_backward, attention_forward, prologue_backward, prologue_forward)
+
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    props = torch.cuda.get_device_properties(dev)
+    wl_cpu = workloads.make(args.workload)
+    wl = wl_cpu.to(dev)
+    sp = wl.spec
+    K, W = args.steps, args.warmup
+
+    # ---- tile map (once per training step in the model; timed on its own) -------------------
+    tmap = build_tile_map(wl.document_ids, sp.B, sp.S, True, sp.window)
+    t_map = time_region(lambda: build_tile_map(wl.document_ids, sp.B, sp.S, True, sp.window), K, W)
+
+    # ---- prologue --------------------------------------------------------------------------
+    q, k, q_rstd, k_rstd = prologue_forward(wl.xq, wl.xk, wl.q_w, wl.k_w, wl.cos, wl.sin, wl.position_ids)
+    t_pro_f = time_region(lambda: prologue_forward(wl.xq, wl.xk, wl.q_w, wl.k_w, wl.cos, wl.sin, wl.position_ids), K, W)
+    elt = wl.xq.element_size()
+    pro_bytes = 2 * elt * sp.B * sp.S * (sp.Hq + sp.Hkv) * sp.D + 8 * sp.B * sp.S + 8 * sp.B * sp.S * (sp.D // 2)
+
+    # ---- attention: the timed step ------------------------------------------------------------
+    out, lse = attention_forward(q, k, wl.xv, tmap, wl.document_ids, wl.scale, True, sp.window)
+    has_bwd = wl.dout is not None
+    bufs = None
+    if has_bwd:
+        dq, dk, dv = attention_backward(q, k, wl.xv, out, wl.dout, lse, tmap, wl.document_ids, wl.scale, True, sp.window)
+        ws = torch.empty(max(_lib.lib().ma_attn_bwd_workspace_bytes(sp.B, sp.S, sp.Hq, sp.Hkv, sp.D), 16),
+                         dtype=torch.uint8, device=dev)
+        bufs = (dq, dk, dv, ws)
+
+    def fwd():
+        return attention_forward(q, k, wl.xv, tmap, wl.document_ids, wl.scale, True, sp.window)
+
+    def bwd(stages=_lib.MA_BWD_ALL):
+        return attention_backward(q, k, wl.xv, out, wl.dout, lse, tmap, wl.document_ids, wl.scale, True, sp.window,
+                                  stages=stages, buffers=bufs)
+
+    def step():
+        fwd()
+        if has_bwd:
+            bwd()
+
+    for _ in range(W):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(K):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / K
+
+    # per-kernel durations, HIP events on the launch stream
+    t_fwd = time_region(fwd, K, W)
+    t_delta = t_dkv = t_dq = t_bwd = None
+    if has_bwd:
+        t_bwd = time_region(bwd, K, W)
+        t_delta = time_region(lambda: bwd(_lib.MA_BWD_DELTA), K, W)
+        t_dkv = time_region(lambda: bwd(_lib.MA_BWD_DKV), K, W)
+        t_dq = time_region(lambda: bwd(_lib.MA_BWD_DQ), K, W)
+        t_pro_b = time_region(
+            lambda: prologue_backward(wl.xq, wl.xk, dq, dk, wl.q_w, wl.k_w, wl.cos, wl.sin, wl.position_ids, q_rstd,
+                                      k_rstd), K, W)
+    # the whole autograd Function (prologue + attention, forward + backward), for reference
+    t_full = None
+    if has_bwd:
+        xs = [wl.xq.clone().requires_grad_(), wl.xk.clone().requires_grad_(), wl.xv.clone().requires_grad_()]
+        ws_ = [None if w is None else w.clone().requires_grad_() for w in (wl.q_w, wl.k_w)]
+
+        def full():
+            o = packed_doc_attention(xs[0], xs[1], xs[2], ws_[0], ws_[1], wl.cos, wl.sin, wl.position_ids,
+                                     wl.document_ids, wl.scale, True, sp.window, 1e-6, tmap)
+            torch.autograd.grad(o, xs + [w for w in ws_ if w is not None], wl.dout)
+        t_full = time_region(full, max(K // 2, 2), 2)
+
+    fl = wl.useful_flops()
+    total_flops = fl["fwd_bwd"] if has_bwd else fl["fwd"]
+    value = total_flops / (ms_per_step * 1e-3) / 1e12
+
+    def tf(flops, ms):
+        return None if ms is None else flops / (ms * 1e-3) / 1e12
+
+    base = sp.D * sp.Hq * wl.n_pairs
+    kern = {
+        "attn_fwd_bf16_kernel": {"ms": t_fwd, "algorithmic_flops": 4 * base},
+        "attn_bwd_dkv_bf16_kernel": {"ms": t_dkv, "algorithmic_flops": 6 * base},   # dP, dV, dK
+        "attn_bwd_dq_bf16_kernel": {"ms": t_dq, "algorithmic_flops": 2 * base},     # dQ
+    }
+    for v in kern.values():
+        v["tflops"] = tf(v["algorithmic_flops"], v["ms"])
+    dom_name = max((n for n in kern if kern[n]["ms"] is not None), key=lambda n: kern[n]["ms"])
+    dom = kern[dom_name]
+    roofline = {
+        "kernel": dom_name, "bound": "mfma", "achieved": dom["tflops"], "peak": PEAK_BF16_DENSE_TFLOPS,
+        "unit": "TFLOP/s", "frac": dom["tflops"] / PEAK_BF16_DENSE_TFLOPS, "traffic": None,
+        "avg_launch_ms": dom["ms"], "algorithmic_flops_per_launch": dom["algorithmic_flops"],
+    }
+    traffic_file = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    if os.path.exists(traffic_file):
+        with open(traffic_file) as f:
+            tr = json.load(f)
+        roofline["traffic"] = tr.get(sp.name, {}).get(dom_name)
+
+    T = (sp.S + 127) // 128
+    n_partial, n_full = int(tmap.kv_num_blocks.sum()), int(tmap.full_kv_num_blocks.sum())
+    result = {
+        "metric": "useful TFLOP/s fwd+bwd doc-masked attn, Gemma3-4B S=8192 bf16; % MFMA peak",
+        "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if sp.dtype == torch.bfloat16 else "f32", "data": "synthetic",
+        "config": {"workload": sp.name, "description": sp.description, "B": sp.B, "S": sp.S, "Hq": sp.Hq,
+                   "Hkv": sp.Hkv, "D": sp.D, "window": sp.window, "n_pairs": wl.n_pairs,
+                   "timed_region": "ma_attn_fwd + ma_attn_bwd (delta, dK/dV, dQ) per step, inputs resident in HBM"},
+        "pct_of_bf16_dense_peak": 100.0 * value / PEAK_BF16_DENSE_TFLOPS,
+        "peak_bf16_dense_tflops": PEAK_BF16_DENSE_TFLOPS, "peak_hbm_gbps": PEAK_HBM_GBPS,
+        "device": props.name, "gcn_arch": getattr(props, "gcnArchName", ""), "cus": props.multi_processor_count,
+        "clock_mhz": getattr(props, "clock_rate", 0) / 1e3,
+        "useful_flops": fl,
+        "fwd": {"ms": t_fwd, "tflops": tf(fl["fwd"], t_fwd), "pct_peak": 100 * tf(fl["fwd"], t_fwd) / PEAK_BF16_DENSE_TFLOPS},
+        "bwd": None if not has_bwd else {"ms": t_bwd, "tflops": tf(fl["bwd"], t_bwd),
+                                         "pct_peak": 100 * tf(fl["bwd"], t_bwd) / PEAK_BF16_DENSE_TFLOPS,
+                                         "delta_ms": t_delta, "dkv_ms": t_dkv, "dq_ms": t_dq},
+        "fwd_bwd_flashattn_convention_tflops": tf(fl["fwd_bwd_flashattn_convention"], ms_per_step) if has_bwd else None,
+        "kernels": kern,
+        "prologue": {"fwd_ms": t_pro_f, "fwd_gbps": pro_bytes / (t_pro_f * 1e-3) / 1e9,
+                     "fwd_frac_hbm_peak": pro_bytes / (t_pro_f * 1e-3) / 1e9 / PEAK_HBM_GBPS,
+                     "algorithmic_bytes": pro_bytes,
+                     "bwd_ms": t_pro_b if has_bwd else None},
+        "tile_map": {"build_ms": t_map, "partial_tiles": n_partial, "full_tiles": n_full, "tiles": sp.B * T * T,
+                     "skipped_tile_ratio": 1.0 - (n_partial + n_full) / float(sp.B * T * T),
+                     "skipped_vs_causal": 1.0 - (n_partial + n_full) / float(sp.B * T * (T + 1) // 2)},
+        "full_autograd_function_ms": t_full,
+        "roofline": roofline,
+    }
+    if not args.no_cpu_baseline and has_bwd:
+        result["cpu_baseline"] = cpu_baseline(wl_cpu)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

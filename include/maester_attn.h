@@ -129,6 +129,21 @@ int ma_attn_bwd(const ma_tensor4* q, const ma_tensor4* k, const ma_tensor4* v, c
                 int64_t window, float scale, void* workspace, size_t workspace_bytes, int dtype,
                 int B, int S, int Hq, int Hkv, int D, void* stream);
 
+/* ma_attn_bwd restricted to a subset of its three kernels, for callers that time or overlap them:
+ * stages is a bit mask of MA_BWD_DELTA (writes delta into the workspace), MA_BWD_DKV (reads delta,
+ * writes dk and dv) and MA_BWD_DQ (reads delta, writes dq).  ma_attn_bwd == all three.  No
+ * counterpart in the reference (its backward is one fused Inductor launch,
+ * torch/_inductor/kernel/flex/templates/flex_backwards.py.jinja). */
+#define MA_BWD_DELTA 1
+#define MA_BWD_DKV 2
+#define MA_BWD_DQ 4
+#define MA_BWD_ALL 7
+int ma_attn_bwd_stages(const ma_tensor4* q, const ma_tensor4* k, const ma_tensor4* v, const ma_tensor4* out,
+                       const ma_tensor4* dout, const float* lse, const ma_tensor4* dq, const ma_tensor4* dk,
+                       const ma_tensor4* dv, const ma_tile_map* map, const int64_t* document_ids, int causal,
+                       int64_t window, float scale, void* workspace, size_t workspace_bytes, int dtype,
+                       int B, int S, int Hq, int Hkv, int D, int stages, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -20,11 +20,12 @@ MA_ERR_LAUNCH = -3
 MA_DTYPE_F32 = 0
 MA_DTYPE_BF16 = 1
 MA_TILE = 128
+MA_BWD_DELTA, MA_BWD_DKV, MA_BWD_DQ, MA_BWD_ALL = 1, 2, 4, 7
 
 EXPORTS = (
     "ma_version", "ma_last_error", "ma_tile_map_workspace_bytes", "ma_tile_map_build", "ma_prologue_fwd",
     "ma_prologue_bwd_workspace_bytes", "ma_prologue_bwd", "ma_attn_fwd", "ma_attn_bwd_workspace_bytes",
-    "ma_attn_bwd",
+    "ma_attn_bwd", "ma_attn_bwd_stages",
 )
 
 
@@ -85,6 +86,8 @@ def lib() -> ctypes.CDLL:
     L.ma_attn_bwd.restype = c_int
     L.ma_attn_bwd.argtypes = [T4, T4, T4, T4, T4, c_void_p, T4, T4, T4, TM, c_void_p, c_int, c_int64, c_float,
                               c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]
+    L.ma_attn_bwd_stages.restype = c_int
+    L.ma_attn_bwd_stages.argtypes = L.ma_attn_bwd.argtypes[:-1] + [c_int, c_void_p]
     _lib = L
     return L
 

@@ -131,26 +131,32 @@ def attention_forward(q, k, v, tile_map: TileMap, document_ids, scale, causal=Tr
     return out, lse
 
 
-def attention_backward(q, k, v, out, dout, lse, tile_map: TileMap, document_ids, scale, causal=True, window=None):
-    """Returns (dq, dk, dv) as new contiguous [B,S,H,D] tensors."""
+def attention_backward(q, k, v, out, dout, lse, tile_map: TileMap, document_ids, scale, causal=True, window=None,
+                       stages=_lib.MA_BWD_ALL, buffers=None):
+    """Returns (dq, dk, dv) as new contiguous [B,S,H,D] tensors.  ``stages`` restricts the call to
+    some of its kernels (see ``ma_attn_bwd_stages``); ``buffers`` = (dq, dk, dv, workspace) reuses
+    tensors from an earlier call, which staged calls need."""
     B, S, Hq, Hkv, D = _check_qkv(q, k, v)
     q, k, v, out, dout = (_rowmajor(t) for t in (q, k, v, out, dout))
     dev = q.device
     L = _lib.lib()
-    dq = torch.empty((B, S, Hq, D), dtype=q.dtype, device=dev)
-    dk = torch.empty((B, S, Hkv, D), dtype=q.dtype, device=dev)
-    dv = torch.empty((B, S, Hkv, D), dtype=q.dtype, device=dev)
     ws_bytes = L.ma_attn_bwd_workspace_bytes(B, S, Hq, Hkv, D)
-    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+    if buffers is None:
+        dq = torch.empty((B, S, Hq, D), dtype=q.dtype, device=dev)
+        dk = torch.empty((B, S, Hkv, D), dtype=q.dtype, device=dev)
+        dv = torch.empty((B, S, Hkv, D), dtype=q.dtype, device=dev)
+        ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+    else:
+        dq, dk, dv, ws = buffers
     doc = _ids(document_ids, B, S, "document_ids")
     cs = tile_map.c_struct()
     with torch.cuda.device(dev):
-        rc = L.ma_attn_bwd(
+        rc = L.ma_attn_bwd_stages(
             byref(_lib.tensor4(q)), byref(_lib.tensor4(k)), byref(_lib.tensor4(v)), byref(_lib.tensor4(out)),
             byref(_lib.tensor4(dout)), _lib.ptr(lse), byref(_lib.tensor4(dq)), byref(_lib.tensor4(dk)),
             byref(_lib.tensor4(dv)), byref(cs), _lib.ptr(doc), 1 if causal else 0,
             -1 if window is None else int(window), float(scale), _lib.ptr(ws), ws_bytes,
-            _lib.dtype_code(q.dtype), B, S, Hq, Hkv, D, _lib.current_stream(dev))
+            _lib.dtype_code(q.dtype), B, S, Hq, Hkv, D, int(stages), _lib.current_stream(dev))
     _lib.check(rc)
     return dq, dk, dv
 

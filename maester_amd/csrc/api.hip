@@ -212,7 +212,17 @@ int ma_attn_bwd(const ma_tensor4* q, const ma_tensor4* k, const ma_tensor4* v, c
                 const ma_tensor4* dv, const ma_tile_map* map, const int64_t* document_ids, int causal, int64_t window,
                 float scale, void* workspace, size_t workspace_bytes, int dtype, int B, int S, int Hq, int Hkv, int D,
                 void* stream) {
+    return ma_attn_bwd_stages(q, k, v, out, dout, lse, dq, dk, dv, map, document_ids, causal, window, scale, workspace,
+                              workspace_bytes, dtype, B, S, Hq, Hkv, D, MA_BWD_ALL, stream);
+}
+
+int ma_attn_bwd_stages(const ma_tensor4* q, const ma_tensor4* k, const ma_tensor4* v, const ma_tensor4* out,
+                       const ma_tensor4* dout, const float* lse, const ma_tensor4* dq, const ma_tensor4* dk,
+                       const ma_tensor4* dv, const ma_tile_map* map, const int64_t* document_ids, int causal,
+                       int64_t window, float scale, void* workspace, size_t workspace_bytes, int dtype, int B, int S,
+                       int Hq, int Hkv, int D, int stages, void* stream) {
     const char* who = "ma_attn_bwd";
+    if (stages <= 0 || (stages & ~MA_BWD_ALL)) return fail(MA_ERR_BAD_ARG, "%s: stages mask %d is invalid", who, stages);
     AttnArgs a;
     MA_TRY(fill_attn(who, a, q, k, v, out, map, document_ids, causal, window, scale, dtype, B, S, Hq, Hkv, D, true));
     MA_TRY(check_tensor(who, "dout", dout, dtype));
@@ -227,6 +237,7 @@ int ma_attn_bwd(const ma_tensor4* q, const ma_tensor4* k, const ma_tensor4* v, c
     a.dout = *dout; a.dq = *dq; a.dk = *dk; a.dv = *dv;
     a.lse = (float*)lse;
     a.delta = (float*)workspace;
+    a.stages = stages;
     return dtype == MA_DTYPE_BF16 ? launch_attn_bwd_bf16(a, (hipStream_t)stream)
                                   : launch_attn_bwd_f32(a, (hipStream_t)stream);
 }

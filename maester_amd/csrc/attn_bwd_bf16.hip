@@ -330,16 +330,22 @@ template <int D>
 static int bwd_d(const AttnArgs& a, hipStream_t st) {
     constexpr int RPB = 256 / (D / 8);
     const int64_t nrows = (int64_t)a.B * a.Hq * a.S;
-    hipLaunchKernelGGL(attn_delta_bf16_kernel<D>, dim3((unsigned)((nrows + RPB - 1) / RPB)), dim3(256), 0, st, a);
-    int rc = check_launch("attn_delta_bf16_kernel");
-    if (rc) return rc;
+    int rc = MA_OK;
+    if (a.stages & MA_BWD_DELTA) {
+        hipLaunchKernelGGL(attn_delta_bf16_kernel<D>, dim3((unsigned)((nrows + RPB - 1) / RPB)), dim3(256), 0, st, a);
+        rc = check_launch("attn_delta_bf16_kernel");
+        if (rc) return rc;
+    }
 
     const size_t lds_kv = (size_t)2 * kStep * D * 2 + kStep * (4 + 4 + 8);
     rc = opt_in_lds(attn_bwd_dkv_bf16_kernel<D>, lds_kv, "attn_bwd_dkv_bf16");
     if (rc) return rc;
-    hipLaunchKernelGGL(attn_bwd_dkv_bf16_kernel<D>, dim3(a.T, a.Hkv, a.B), dim3(kBwdThreads), lds_kv, st, a);
-    rc = check_launch("attn_bwd_dkv_bf16_kernel");
-    if (rc) return rc;
+    if (a.stages & MA_BWD_DKV) {
+        hipLaunchKernelGGL(attn_bwd_dkv_bf16_kernel<D>, dim3(a.T, a.Hkv, a.B), dim3(kBwdThreads), lds_kv, st, a);
+        rc = check_launch("attn_bwd_dkv_bf16_kernel");
+        if (rc) return rc;
+    }
+    if (!(a.stages & MA_BWD_DQ)) return MA_OK;
 
     const size_t lds_q = (size_t)2 * kStep * D * 2 + kStep * 8;
     rc = opt_in_lds(attn_bwd_dq_bf16_kernel<D>, lds_q, "attn_bwd_dq_bf16");

@@ -330,15 +330,21 @@ template <int D>
 static int bwd_d(const AttnArgs& a, hipStream_t st) {
     using C = F32Cfg<D>;
     const int64_t nrows = (int64_t)a.B * a.Hq * a.S;
-    hipLaunchKernelGGL(attn_delta_f32_kernel, dim3((unsigned)((nrows + 255) / 256)), dim3(256), 0, st, a);
-    int rc = check_launch("attn_delta_f32_kernel");
-    if (rc) return rc;
+    int rc = MA_OK;
+    if (a.stages & MA_BWD_DELTA) {
+        hipLaunchKernelGGL(attn_delta_f32_kernel, dim3((unsigned)((nrows + 255) / 256)), dim3(256), 0, st, a);
+        rc = check_launch("attn_delta_f32_kernel");
+        if (rc) return rc;
+    }
     const size_t lds_q = (size_t)(2 * kRows * C::LDQ + 2 * C::KC * D) * 4 + C::KC * 8;
     rc = set_lds(attn_bwd_dq_f32_kernel<D>, lds_q);
     if (rc) return rc;
-    hipLaunchKernelGGL(attn_bwd_dq_f32_kernel<D>, dim3(2 * a.T, a.Hq, a.B), dim3(kRows), lds_q, st, a);
-    rc = check_launch("attn_bwd_dq_f32_kernel");
-    if (rc) return rc;
+    if (a.stages & MA_BWD_DQ) {
+        hipLaunchKernelGGL(attn_bwd_dq_f32_kernel<D>, dim3(2 * a.T, a.Hq, a.B), dim3(kRows), lds_q, st, a);
+        rc = check_launch("attn_bwd_dq_f32_kernel");
+        if (rc) return rc;
+    }
+    if (!(a.stages & MA_BWD_DKV)) return MA_OK;
     const size_t lds_k = (size_t)(2 * kRows * (D + 1) + 2 * 16 * D + 32) * 4 + 16 * 8;
     rc = set_lds(attn_bwd_dkv_f32_kernel<D>, lds_k);
     if (rc) return rc;

@@ -53,6 +53,7 @@ struct AttnArgs {
     int64_t window;
     float scale;
     int B, S, Hq, Hkv, D, T;
+    int stages;  // MA_BWD_* mask (backward only)
 };
 
 int launch_attn_fwd_f32(const AttnArgs& a, hipStream_t st);

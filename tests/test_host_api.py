@@ -1,0 +1,157 @@
+"""CPU-side checks: the C-ABI library loads, exports every symbol the header declares, and rejects
+bad arguments before any launch; workload generators reproduce the survey's census."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from maester_amd import _lib, workloads
+from maester_amd._lib import MaTensor4, MaTileMap
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "maester_attn.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ma_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    L = _lib.lib()
+    names = _declared_symbols()
+    assert set(names) == set(_lib.EXPORTS), (names, _lib.EXPORTS)
+    for n in names:
+        assert hasattr(L, n), n
+    assert L.ma_version() >= 100
+    assert L.ma_last_error() is not None
+
+
+def _t4(ptr=0x1000, sb=1 << 20, ss=1024, sh=256):
+    return MaTensor4(ptr, sb, ss, sh)
+
+
+def _map(ok=True):
+    return MaTileMap(*([0x1000] * 8 if ok else [0] * 8))
+
+
+def _err():
+    return _lib.lib().ma_last_error().decode()
+
+
+def test_workspace_sizes():
+    L = _lib.lib()
+    assert L.ma_tile_map_workspace_bytes(4, 8192) == 4 * 64 * 64
+    assert L.ma_tile_map_workspace_bytes(1, 129) == 4
+    assert L.ma_tile_map_workspace_bytes(0, 10) == 0
+    assert L.ma_attn_bwd_workspace_bytes(4, 8192, 8, 4, 256) == 4 * 8 * 8192 * 4
+    assert L.ma_prologue_bwd_workspace_bytes(4, 8192, 8, 4, 256) > 0
+
+
+def test_tile_map_argument_errors():
+    L = _lib.lib()
+    m = _map()
+    assert L.ma_tile_map_build(None, 0, 128, 1, -1, ctypes.byref(m), 0x1000, 1 << 20, None) == _lib.MA_ERR_BAD_ARG
+    assert "positive" in _err()
+    assert L.ma_tile_map_build(None, 1, 128, 2, -1, ctypes.byref(m), 0x1000, 1 << 20, None) == _lib.MA_ERR_BAD_ARG
+    assert L.ma_tile_map_build(None, 1, 128, 1, -5, ctypes.byref(m), 0x1000, 1 << 20, None) == _lib.MA_ERR_BAD_ARG
+    assert "window" in _err()
+    assert L.ma_tile_map_build(None, 1, 128, 1, -1, None, 0x1000, 1 << 20, None) == _lib.MA_ERR_BAD_ARG
+    bad = _map(False)
+    assert L.ma_tile_map_build(None, 1, 128, 1, -1, ctypes.byref(bad), 0x1000, 1 << 20, None) == _lib.MA_ERR_BAD_ARG
+    assert L.ma_tile_map_build(None, 1, 1024, 1, -1, ctypes.byref(m), 0x1000, 8, None) == _lib.MA_ERR_BAD_ARG
+    assert "workspace" in _err()
+    assert L.ma_tile_map_build(None, 1, 1024, 1, -1, ctypes.byref(m), None, 1 << 20, None) == _lib.MA_ERR_BAD_ARG
+
+
+def test_attention_argument_errors():
+    L = _lib.lib()
+    t, m = _t4(), _map()
+    r = ctypes.byref
+
+    def fwd(q=t, k=t, v=t, o=t, lse=0x1000, mp=m, causal=1, window=-1, scale=0.1, dtype=1, B=1, S=256, Hq=4, Hkv=2, D=256):
+        return L.ma_attn_fwd(r(q), r(k), r(v), r(o), lse, r(mp), None, causal, window, scale, dtype, B, S, Hq, Hkv, D, None)
+
+    assert fwd(D=96) == _lib.MA_ERR_UNSUPPORTED and "head_dim" in _err()
+    assert fwd(Hq=5) == _lib.MA_ERR_BAD_ARG and "multiple" in _err()
+    assert fwd(dtype=7) == _lib.MA_ERR_BAD_ARG
+    assert fwd(scale=0.0) == _lib.MA_ERR_BAD_ARG and "scale" in _err()
+    assert fwd(scale=float("nan")) == _lib.MA_ERR_BAD_ARG
+    assert fwd(lse=None) == _lib.MA_ERR_BAD_ARG and "lse" in _err()
+    assert fwd(q=_t4(ptr=0)) == _lib.MA_ERR_BAD_ARG and "NULL" in _err()
+    assert fwd(q=_t4(ptr=0x1004)) == _lib.MA_ERR_BAD_ARG and "aligned" in _err()
+    assert fwd(k=_t4(ss=1023)) == _lib.MA_ERR_BAD_ARG and "strides" in _err()
+    assert fwd(mp=_map(False)) == _lib.MA_ERR_BAD_ARG and "tile map" in _err()
+    assert fwd(causal=3) == _lib.MA_ERR_BAD_ARG
+    assert fwd(B=0) == _lib.MA_ERR_BAD_ARG
+    # backward: workspace too small, invalid stages
+    rc = L.ma_attn_bwd(r(t), r(t), r(t), r(t), r(t), 0x1000, r(t), r(t), r(t), r(m), None, 1, -1, 0.1, 0x1000, 16, 1,
+                       1, 256, 4, 2, 256, None)
+    assert rc == _lib.MA_ERR_BAD_ARG and "workspace" in _err()
+    rc = L.ma_attn_bwd_stages(r(t), r(t), r(t), r(t), r(t), 0x1000, r(t), r(t), r(t), r(m), None, 1, -1, 0.1, 0x1000,
+                              1 << 30, 1, 1, 256, 4, 2, 256, 9, None)
+    assert rc == _lib.MA_ERR_BAD_ARG and "stages" in _err()
+
+
+def test_prologue_argument_errors():
+    L = _lib.lib()
+    t = _t4()
+    r = ctypes.byref
+    rc = L.ma_prologue_fwd(r(t), r(t), r(t), r(t), None, None, None, 0x1000, 100, None, 1e-6, 1, None, None, 1, 1, 64, 4,
+                           2, 256, None)
+    assert rc == _lib.MA_ERR_BAD_ARG and "rope" in _err()
+    rc = L.ma_prologue_fwd(r(t), r(t), r(t), r(t), None, None, 0x1000, 0x1000, 10, None, 1e-6, 1, None, None, 1, 1, 64,
+                           4, 2, 256, None)
+    assert rc == _lib.MA_ERR_BAD_ARG and "n_pos" in _err()
+    rc = L.ma_prologue_fwd(r(t), r(t), r(t), r(t), 0x1000, None, 0x1000, 0x1000, 100, None, 1e-6, 1, None, None, 1, 1,
+                           64, 4, 2, 256, None)
+    assert rc == _lib.MA_ERR_BAD_ARG and "q_rstd" in _err()
+    rc = L.ma_prologue_fwd(r(t), r(t), r(t), r(t), None, None, 0x1000, 0x1000, 100, None, 1e-6, 1, None, None, 1, 1, 64,
+                           4, 2, 100, None)
+    assert rc == _lib.MA_ERR_UNSUPPORTED
+
+
+def test_python_front_end_refuses_cpu_tensors():
+    from maester_amd import build_tile_map, doc_masked_attention
+    q = torch.zeros(1, 128, 2, 64)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        doc_masked_attention(q, q, q, torch.zeros(1, 128, dtype=torch.long))
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        build_tile_map(torch.zeros(1, 128, dtype=torch.long), 1, 128)
+    with pytest.raises(TypeError):
+        _lib.dtype_code(torch.float16)
+
+
+def test_workload_census_matches_survey():
+    want = {"c1": 278607, "c2": 21977636, "c3": 17311446, "c4": 138550011, "c5": 44817787}
+    for name, pairs in want.items():
+        sp = workloads.spec(name)
+        rows = workloads.document_lengths(sp)
+        assert all(sum(r) == sp.S for r in rows)
+        assert workloads.count_pairs(rows, sp.window) == pairs
+    # the closed form equals a brute-force count on a small window case
+    from oracle import tile_map as otm
+    wl = workloads.make("c3", B=2, S=2048)
+    assert wl.n_pairs == otm.count_pairs(wl.document_ids.numpy(), 2, 2048, True, 1024)
+    assert (wl.position_ids[wl.document_ids == 0][:5] == torch.arange(5)).all()
+    assert wl.xq.dtype == torch.bfloat16 and wl.q_w.shape == (256,)
+    wlp = workloads.make("c2", B=1, S=1024, pad_tail=100)
+    assert (wlp.document_ids[:, -100:] == -1).all() and (wlp.position_ids[:, -100:] == 0).all()
+
+
+def test_gemma_module_mirrors_reference_interface():
+    from maester_amd import GemmaAttention, GemmaAttentionConfig
+    cfg = GemmaAttentionConfig(dim=64, n_heads=2, num_key_value_heads=1, head_dim=64, max_seq_len=128,
+                               sliding_window_size=32, query_pre_attn_scalar=256)
+    attn = GemmaAttention(cfg, "local_sliding")
+    assert attn.scaling == 256 ** -0.5
+    assert attn.rope_cos.shape == (256, 32)
+    assert set(dict(attn.named_parameters())) == {"qkv_proj.weight", "o_proj.weight", "query_norm.weight", "key_norm.weight"}
+    assert float(attn.query_norm.weight.abs().sum()) == 0.0          # zeros-initialised, scale 1+w
+    with pytest.raises(ValueError):
+        attn.set_backend("triton")
+    with pytest.raises(NotImplementedError):
+        attn.set_backend("flex")
+    attn.set_backend("hip")
