@@ -53,19 +53,22 @@ __global__ __launch_bounds__(256) void attn_delta_bf16_kernel(AttnArgs a) {
 // ------------------------------------------------------------------------------------------------
 template <int D>
 __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dkv_bf16_kernel(AttnArgs a) {
+    using TL = Tile<D>;
     constexpr int KK = D / 16;
     constexpr int DB = D / 32;
     constexpr int BM = kStep;
     extern __shared__ __align__(16) char smem_raw[];
     lds_ptr Qs = (lds_ptr)smem_raw;
-    lds_ptr Gs = Qs + BM * D * 2;  // dO rows
-    MA_LDS float* lse2s = (MA_LDS float*)(Gs + BM * D * 2);
+    lds_ptr Gs = Qs + TL::bytes(BM);  // dO rows
+    MA_LDS float* lse2s = (MA_LDS float*)(Gs + TL::bytes(BM));
     MA_LDS float* dls = lse2s + BM;
     MA_LDS int64_t* qdoc = (MA_LDS int64_t*)(dls + BM);
 
-    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 31, hh = lane >> 5;
-    const int j = blockIdx.x, hk = blockIdx.y, b = blockIdx.z;
+    const int j = blockIdx.y, hk = blockIdx.x % a.Hkv, b = blockIdx.x / a.Hkv;
+    const int rbase = TL::row_base(lane), tbase = TL::tr_base(lane);
     const int G = a.Hq / a.Hkv;
     const int kw_lo = j * kTile + 32 * w, kw_hi = kw_lo + 31;
     const int kv = kw_lo + r;
@@ -77,18 +80,16 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dkv_bf16_kernel(AttnArgs
     const __bf16* vp = (const __bf16*)a.v.ptr + b * a.v.stride_b + hk * a.v.stride_h;
     const int64_t* drow = a.doc ? a.doc + (size_t)b * a.S : nullptr;
 
+    // rows past the end of the sequence read the last valid row; their results are masked / not stored
+    const int kvc = min(kv, a.S - 1);
     bf16x8 kf[KK], vf[KK];
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
-        bf16x8 zk = {0, 0, 0, 0, 0, 0, 0, 0}, zv = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (kvalid) {
-            zk = *(const bf16x8*)(kp + (int64_t)kv * a.k.stride_s + 16 * kk + 8 * hh);
-            zv = *(const bf16x8*)(vp + (int64_t)kv * a.v.stride_s + 16 * kk + 8 * hh);
-        }
-        kf[kk] = zk;
-        vf[kk] = zv;
+        kf[kk] = *(const bf16x8*)(kp + (int64_t)kvc * a.k.stride_s + 16 * kk + 8 * hh);
+        vf[kk] = *(const bf16x8*)(vp + (int64_t)kvc * a.v.stride_s + 16 * kk + 8 * hh);
     }
-    const int64_t dock = (drow && kvalid) ? drow[kv] : 0;
+    const int64_t dock = drow ? drow[kvc] : 0;
+    const int wlim = a.window >= 0 ? (int)min(a.window, (int64_t)0x3fffffff) : 0x7fffffff;
 
     f32x16 dkacc[DB], dvacc[DB];
 #pragma unroll
@@ -118,8 +119,13 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dkv_bf16_kernel(AttnArgs
 
                 __syncthreads();
                 const int rows_valid = min(BM, a.S - q0);
-                stage_tile<D, BM, kBwdThreads>(Qs, qp + (int64_t)q0 * a.q.stride_s, a.q.stride_s, rows_valid, tid);
-                stage_tile<D, BM, kBwdThreads>(Gs, gp + (int64_t)q0 * a.dout.stride_s, a.dout.stride_s, rows_valid, tid);
+                {
+                    Stager<D, BM, kBwdThreads> sq, sg;
+                    sq.load(qp + (int64_t)q0 * a.q.stride_s, a.q.stride_s, rows_valid, tid);
+                    sg.load(gp + (int64_t)q0 * a.dout.stride_s, a.dout.stride_s, rows_valid, tid);
+                    sq.store(Qs, rows_valid, tid);
+                    sg.store(Gs, rows_valid, tid);
+                }
                 if (tid < BM) {
                     const bool ok = q0 + tid < a.S;
                     lse2s[tid] = ok ? a.lse[rowbase + q0 + tid] * kLog2e : 0.f;
@@ -139,19 +145,24 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dkv_bf16_kernel(AttnArgs
 #pragma unroll
                     for (int v = 0; v < 16; ++v) s[v] = dp[v] = 0.f;
 #pragma unroll
-                    for (int kk = 0; kk < KK; ++kk) s = mfma32(row_frag<D>(Qs, 32 * mb + r, 2 * kk + hh), kf[kk], s);
+                    for (int kk = 0; kk < KK; ++kk) s = mfma32(TL::row_frag(Qs, rbase, 32 * mb, kk), kf[kk], s);
 #pragma unroll
-                    for (int kk = 0; kk < KK; ++kk) dp = mfma32(row_frag<D>(Gs, 32 * mb + r, 2 * kk + hh), vf[kk], dp);
+                    for (int kk = 0; kk < KK; ++kk) dp = mfma32(TL::row_frag(Gs, rbase, 32 * mb, kk), vf[kk], dp);
 
                     bf16x8 pf[2], dsf[2];
+                    // d = q - kv for element v is drel + 8*(v/4) + v%4; all tests are branch-free
+                    const int drel = q0 + 32 * mb + 4 * hh - kv;
+                    const int dmin = bounded ? 0 : -0x40000000;
+                    const int dend = a.S - kv;                    // q < S  <=>  d < S - kv
 #pragma unroll
                     for (int v = 0; v < 16; ++v) {
-                        const int ql = 32 * mb + 8 * (v >> 2) + 4 * hh + (v & 3);
+                        const int qc = 8 * (v >> 2) + (v & 3);
+                        const int ql = 32 * mb + qc + 4 * hh;
                         float p = fast_exp2(s[v] * sl2 - lse2s[ql]);
                         if (partial) {
-                            const int qq = q0 + ql;
-                            bool ok = kvalid && qq < a.S && pair_allowed(qq, kv, a.causal, a.window);
-                            if (drow) ok = ok && (qdoc[ql] == dock);
+                            const int d = drel + qc;
+                            bool ok = (d >= dmin) & (d <= wlim) & (d < dend) & kvalid;
+                            if (drow) ok = ok & (qdoc[ql] == dock);
                             p = ok ? p : 0.f;
                         }
                         const float ds = p * (dp[v] - dls[ql]);
@@ -162,8 +173,8 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dkv_bf16_kernel(AttnArgs
                     for (int t = 0; t < 2; ++t) {
 #pragma unroll
                         for (int db = 0; db < DB; ++db) {
-                            dvacc[db] = mfma32(tr_frag<D>(Gs, 32 * mb + 16 * t, 32 * db, lane), pf[t], dvacc[db]);
-                            dkacc[db] = mfma32(tr_frag<D>(Qs, 32 * mb + 16 * t, 32 * db, lane), dsf[t], dkacc[db]);
+                            dvacc[db] = mfma32(TL::tr_frag(Gs, tbase, 32 * mb + 16 * t, 32 * db), pf[t], dvacc[db]);
+                            dkacc[db] = mfma32(TL::tr_frag(Qs, tbase, 32 * mb + 16 * t, 32 * db), dsf[t], dkacc[db]);
                         }
                     }
                 }
@@ -196,18 +207,21 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dkv_bf16_kernel(AttnArgs
 // ------------------------------------------------------------------------------------------------
 template <int D>
 __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dq_bf16_kernel(AttnArgs a) {
+    using TL = Tile<D>;
     constexpr int KK = D / 16;
     constexpr int DB = D / 32;
     constexpr int BN = kStep;
     extern __shared__ __align__(16) char smem_raw[];
     lds_ptr Ks = (lds_ptr)smem_raw;
-    lds_ptr Vs = Ks + BN * D * 2;
-    MA_LDS int64_t* kdoc = (MA_LDS int64_t*)(Vs + BN * D * 2);
+    lds_ptr Vs = Ks + TL::bytes(BN);
+    MA_LDS int64_t* kdoc = (MA_LDS int64_t*)(Vs + TL::bytes(BN));
 
-    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 31, hh = lane >> 5;
-    const int i = gridDim.x - 1 - blockIdx.x;
-    const int h = blockIdx.y, b = blockIdx.z;
+    const int i = gridDim.y - 1 - blockIdx.y;
+    const int h = blockIdx.x % a.Hq, b = blockIdx.x / a.Hq;
+    const int rbase = TL::row_base(lane), tbase = TL::tr_base(lane);
     const int hk = h / (a.Hq / a.Hkv);
     const int qw_lo = i * kTile + 32 * w, qw_hi = qw_lo + 31;
     const int q = qw_lo + r;
@@ -221,19 +235,16 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dq_bf16_kernel(AttnArgs 
     const __bf16* vp = (const __bf16*)a.v.ptr + b * a.v.stride_b + hk * a.v.stride_h;
     const int64_t* drow = a.doc ? a.doc + (size_t)b * a.S : nullptr;
 
+    const int qc = min(q, a.S - 1);  // rows past the end read the last valid row; never stored
     bf16x8 qf[KK], gf[KK];
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
-        bf16x8 zq = {0, 0, 0, 0, 0, 0, 0, 0}, zg = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (qvalid) {
-            zq = *(const bf16x8*)(qp + (int64_t)q * a.q.stride_s + 16 * kk + 8 * hh);
-            zg = *(const bf16x8*)(gp + (int64_t)q * a.dout.stride_s + 16 * kk + 8 * hh);
-        }
-        qf[kk] = zq;
-        gf[kk] = zg;
+        qf[kk] = *(const bf16x8*)(qp + (int64_t)qc * a.q.stride_s + 16 * kk + 8 * hh);
+        gf[kk] = *(const bf16x8*)(gp + (int64_t)qc * a.dout.stride_s + 16 * kk + 8 * hh);
     }
-    const int64_t docq = (drow && qvalid) ? drow[q] : 0;
-    const size_t rowi = ((size_t)b * a.Hq + h) * a.S + (qvalid ? q : 0);
+    const int64_t docq = drow ? drow[qc] : 0;
+    const int wlim = a.window >= 0 ? (int)min(a.window, (int64_t)0x3fffffff) : 0x7fffffff;
+    const size_t rowi = ((size_t)b * a.Hq + h) * a.S + qc;
     const float lse2 = a.lse[rowi] * kLog2e;
     const float delta = a.delta[rowi];
 
@@ -260,8 +271,13 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dq_bf16_kernel(AttnArgs 
 
             __syncthreads();
             const int rows_valid = min(BN, a.S - k0);
-            stage_tile<D, BN, kBwdThreads>(Ks, kp + (int64_t)k0 * a.k.stride_s, a.k.stride_s, rows_valid, tid);
-            stage_tile<D, BN, kBwdThreads>(Vs, vp + (int64_t)k0 * a.v.stride_s, a.v.stride_s, rows_valid, tid);
+            {
+                Stager<D, BN, kBwdThreads> sk, sv;
+                sk.load(kp + (int64_t)k0 * a.k.stride_s, a.k.stride_s, rows_valid, tid);
+                sv.load(vp + (int64_t)k0 * a.v.stride_s, a.v.stride_s, rows_valid, tid);
+                sk.store(Ks, rows_valid, tid);
+                sv.store(Vs, rows_valid, tid);
+            }
             if (partial && drow && tid < BN) kdoc[tid] = (k0 + tid < a.S) ? drow[k0 + tid] : 0;
             __syncthreads();
 
@@ -276,19 +292,22 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dq_bf16_kernel(AttnArgs 
 #pragma unroll
                 for (int v = 0; v < 16; ++v) s[v] = dp[v] = 0.f;
 #pragma unroll
-                for (int kk = 0; kk < KK; ++kk) s = mfma32(row_frag<D>(Ks, 32 * nb + r, 2 * kk + hh), qf[kk], s);
+                for (int kk = 0; kk < KK; ++kk) s = mfma32(TL::row_frag(Ks, rbase, 32 * nb, kk), qf[kk], s);
 #pragma unroll
-                for (int kk = 0; kk < KK; ++kk) dp = mfma32(row_frag<D>(Vs, 32 * nb + r, 2 * kk + hh), gf[kk], dp);
+                for (int kk = 0; kk < KK; ++kk) dp = mfma32(TL::row_frag(Vs, rbase, 32 * nb, kk), gf[kk], dp);
 
                 bf16x8 dsf[2];
+                const int qrel = q - k0 - 32 * nb - 4 * hh;   // d = q - kv = qrel - (8*(v/4) + v%4)
+                const int dmin = bounded ? 0 : -0x40000000;
+                const int dend = q - a.S;                       // kv < S  <=>  d > q - S
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     float p = fast_exp2(s[v] * sl2 - lse2);
                     if (partial) {
-                        const int kl = 32 * nb + 8 * (v >> 2) + 4 * hh + (v & 3);
-                        const int kvi = k0 + kl;
-                        bool ok = qvalid && kvi < a.S && pair_allowed(q, kvi, a.causal, a.window);
-                        if (drow) ok = ok && (kdoc[kl] == docq);
+                        const int kc = 8 * (v >> 2) + (v & 3);
+                        const int d = qrel - kc;
+                        bool ok = (d >= dmin) & (d <= wlim) & (d > dend) & qvalid;
+                        if (drow) ok = ok & (kdoc[32 * nb + kc + 4 * hh] == docq);
                         p = ok ? p : 0.f;
                     }
                     dsf[v >> 3][v & 7] = (__bf16)(p * (dp[v] - delta));
@@ -297,7 +316,7 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dq_bf16_kernel(AttnArgs 
                 for (int t = 0; t < 2; ++t) {
 #pragma unroll
                     for (int db = 0; db < DB; ++db)
-                        acc[db] = mfma32(tr_frag<D>(Ks, 32 * nb + 16 * t, 32 * db, lane), dsf[t], acc[db]);
+                        acc[db] = mfma32(TL::tr_frag(Ks, tbase, 32 * nb + 16 * t, 32 * db), dsf[t], acc[db]);
                 }
             }
         }
@@ -337,20 +356,20 @@ static int bwd_d(const AttnArgs& a, hipStream_t st) {
         if (rc) return rc;
     }
 
-    const size_t lds_kv = (size_t)2 * kStep * D * 2 + kStep * (4 + 4 + 8);
+    const size_t lds_kv = (size_t)2 * Tile<D>::bytes(kStep) + kStep * (4 + 4 + 8);
     rc = opt_in_lds(attn_bwd_dkv_bf16_kernel<D>, lds_kv, "attn_bwd_dkv_bf16");
     if (rc) return rc;
     if (a.stages & MA_BWD_DKV) {
-        hipLaunchKernelGGL(attn_bwd_dkv_bf16_kernel<D>, dim3(a.T, a.Hkv, a.B), dim3(kBwdThreads), lds_kv, st, a);
+        hipLaunchKernelGGL(attn_bwd_dkv_bf16_kernel<D>, dim3(a.B * a.Hkv, a.T, 1), dim3(kBwdThreads), lds_kv, st, a);
         rc = check_launch("attn_bwd_dkv_bf16_kernel");
         if (rc) return rc;
     }
     if (!(a.stages & MA_BWD_DQ)) return MA_OK;
 
-    const size_t lds_q = (size_t)2 * kStep * D * 2 + kStep * 8;
+    const size_t lds_q = (size_t)2 * Tile<D>::bytes(kStep) + kStep * 8;
     rc = opt_in_lds(attn_bwd_dq_bf16_kernel<D>, lds_q, "attn_bwd_dq_bf16");
     if (rc) return rc;
-    hipLaunchKernelGGL(attn_bwd_dq_bf16_kernel<D>, dim3(a.T, a.Hq, a.B), dim3(kBwdThreads), lds_q, st, a);
+    hipLaunchKernelGGL(attn_bwd_dq_bf16_kernel<D>, dim3(a.B * a.Hq, a.T, 1), dim3(kBwdThreads), lds_q, st, a);
     return check_launch("attn_bwd_dq_bf16_kernel");
 }
 

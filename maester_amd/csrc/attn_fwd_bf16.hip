@@ -5,8 +5,9 @@
 //
 // One workgroup (4 waves) owns a 128-row q tile of one (batch row, q head); wave w owns rows
 // 32w..32w+31 and keeps their Q fragments, the fp32 O^T accumulator and the online-softmax state in
-// registers.  K/V are walked 64 rows at a time through swizzled LDS tiles, following the kv lists
-// of the tile map (partial tiles first, then full tiles -- fully masked tiles are never touched).
+// registers.  K/V are walked 64 rows at a time through LDS tiles, following the kv lists of the
+// tile map (partial tiles first, then full tiles -- fully masked tiles are never touched); the
+// global loads of step n+1 are in flight while step n is computed.
 // Per step:  S^T = K Q^T (MFMA 32x32x16, K row fragments x Q registers), fp32 online softmax in
 // the exp2 domain with the lane owning one q row (row max/sum = in-lane reduction + one 32-lane
 // exchange), P^T cast to bf16 in place, O^T += V^T P^T (MFMA, V through transposed LDS reads).
@@ -20,20 +21,50 @@ namespace ma {
 constexpr int kFwdThreads = 256;
 constexpr int kFwdBN = 64;  // kv rows per step
 
+// Walks the (partial, then full) kv tile lists of one q tile in steps of BN rows, skipping the
+// steps no row of the workgroup can see.  All state is workgroup-uniform.
+struct KvSteps {
+    const int32_t *plist, *flist;
+    int np, nf, it, half, S, q_lo, q_hi, bounded;
+    int64_t window;
+    int k0;
+    bool partial;
+
+    __device__ __forceinline__ bool next() {
+        for (;;) {
+            if (++half == kTile / kFwdBN) {
+                half = 0;
+                ++it;
+            }
+            if (it >= np + nf) return false;
+            partial = it < np;
+            const int j = partial ? plist[it] : flist[it - np];
+            k0 = j * kTile + half * kFwdBN;
+            if (k0 >= S) continue;
+            if (partial && bounded && k0 > q_hi) continue;
+            if (partial && window >= 0 && (int64_t)q_lo - (k0 + kFwdBN - 1) > window) continue;
+            return true;
+        }
+    }
+};
+
 template <int D>
 __global__ __launch_bounds__(kFwdThreads) void attn_fwd_bf16_kernel(AttnArgs a) {
+    using TL = Tile<D>;
     constexpr int KK = D / 16;  // contraction steps of S^T
     constexpr int DB = D / 32;  // 32-row blocks of O^T
     constexpr int BN = kFwdBN;
     extern __shared__ __align__(16) char smem_raw[];
     lds_ptr Ks = (lds_ptr)smem_raw;
-    lds_ptr Vs = Ks + BN * D * 2;
-    MA_LDS int64_t* kdoc = (MA_LDS int64_t*)(Vs + BN * D * 2);
+    lds_ptr Vs = Ks + TL::bytes(BN);
+    MA_LDS int64_t* kdoc = (MA_LDS int64_t*)(Vs + TL::bytes(BN));
 
-    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keep it in a scalar register
     const int r = lane & 31, hh = lane >> 5;
-    const int i = gridDim.x - 1 - blockIdx.x;  // late q tiles see the most keys: start them first
-    const int h = blockIdx.y, b = blockIdx.z;
+    // x walks (batch row, head), y walks q tiles from the last (most keys under causality) to the first
+    const int i = gridDim.y - 1 - blockIdx.y;
+    const int h = blockIdx.x % a.Hq, b = blockIdx.x / a.Hq;
     const int hk = h / (a.Hq / a.Hkv);
     const int qw_lo = i * kTile + 32 * w, qw_hi = qw_lo + 31;
     const int q = qw_lo + r;
@@ -45,14 +76,13 @@ __global__ __launch_bounds__(kFwdThreads) void attn_fwd_bf16_kernel(AttnArgs a) 
     const __bf16* vp = (const __bf16*)a.v.ptr + b * a.v.stride_b + hk * a.v.stride_h;
     const int64_t* drow = a.doc ? a.doc + (size_t)b * a.S : nullptr;
 
+    // rows past the end of the sequence read the last valid row; their results are never stored
+    const int qc = min(q, a.S - 1);
     bf16x8 qf[KK];
 #pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-        bf16x8 val = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (qvalid) val = *(const bf16x8*)(qp + (int64_t)q * a.q.stride_s + 16 * kk + 8 * hh);
-        qf[kk] = val;
-    }
-    const int64_t docq = (drow && qvalid) ? drow[q] : 0;
+    for (int kk = 0; kk < KK; ++kk) qf[kk] = *(const bf16x8*)(qp + (int64_t)qc * a.q.stride_s + 16 * kk + 8 * hh);
+    const int64_t docq = drow ? drow[qc] : 0;
+    const int wlim = a.window >= 0 ? (int)min(a.window, (int64_t)0x3fffffff) : 0x7fffffff;
 
     f32x16 o[DB];
 #pragma unroll
@@ -61,104 +91,141 @@ __global__ __launch_bounds__(kFwdThreads) void attn_fwd_bf16_kernel(AttnArgs a) 
         for (int v = 0; v < 16; ++v) o[db][v] = 0.f;
     float m = -INFINITY, lsum = 0.f;
     const float sl2 = a.scale * kLog2e;
+    const int rbase = TL::row_base(lane), tbase = TL::tr_base(lane);
 
     const size_t mrow = (size_t)b * a.T + i;
-    const int32_t* plist = a.map.kv_indices + mrow * a.T;
-    const int32_t* flist = a.map.full_kv_indices + mrow * a.T;
-    const int np = a.map.kv_num_blocks[mrow];
-    const int nf = a.map.full_kv_num_blocks[mrow];
+    KvSteps st;
+    st.plist = a.map.kv_indices + mrow * a.T;
+    st.flist = a.map.full_kv_indices + mrow * a.T;
+    st.np = a.map.kv_num_blocks[mrow];
+    st.nf = a.map.full_kv_num_blocks[mrow];
+    st.it = 0; st.half = -1; st.S = a.S; st.q_lo = i * kTile; st.q_hi = i * kTile + kTile - 1;
+    st.bounded = bounded; st.window = a.window;
 
-    for (int it = 0; it < np + nf; ++it) {
-        const bool partial = it < np;
-        const int j = partial ? plist[it] : flist[it - np];
-        for (int half = 0; half < kTile / BN; ++half) {
-            const int k0 = j * kTile + half * BN;
-            // steps no row of the workgroup can see (uniform over the workgroup)
-            if (k0 >= a.S) continue;
-            if (partial && bounded && k0 > i * kTile + kTile - 1) continue;
-            if (partial && a.window >= 0 && (int64_t)(i * kTile) - (k0 + BN - 1) > a.window) continue;
+    Stager<D, BN, kFwdThreads> sk, sv;
+    int64_t kd_next = 0;
+    bool have = st.next();
+    int k0 = st.k0, rows_valid = 0;
+    bool partial = st.partial;
+    if (have) {
+        rows_valid = min(BN, a.S - k0);
+        sk.load(kp + (int64_t)k0 * a.k.stride_s, a.k.stride_s, rows_valid, tid);
+        sv.load(vp + (int64_t)k0 * a.v.stride_s, a.v.stride_s, rows_valid, tid);
+        if (partial && drow && tid < BN) kd_next = drow[min(k0 + tid, a.S - 1)];
+    }
 
-            __syncthreads();
-            const int rows_valid = min(BN, a.S - k0);
-            stage_tile<D, BN, kFwdThreads>(Ks, kp + (int64_t)k0 * a.k.stride_s, a.k.stride_s, rows_valid, tid);
-            stage_tile<D, BN, kFwdThreads>(Vs, vp + (int64_t)k0 * a.v.stride_s, a.v.stride_s, rows_valid, tid);
-            if (partial && drow && tid < BN) kdoc[tid] = (k0 + tid < a.S) ? drow[k0 + tid] : 0;
-            __syncthreads();
+    while (have) {
+        __syncthreads();  // everyone is done reading the previous tiles
+        sk.store(Ks, rows_valid, tid);
+        sv.store(Vs, rows_valid, tid);
+        if (partial && drow && tid < BN) kdoc[tid] = kd_next;
+        __syncthreads();
 
-            bool act[2];
+        const int ck0 = k0;
+        const bool cpartial = partial;
+        have = st.next();
+        if (have) {
+            k0 = st.k0;
+            partial = st.partial;
+            rows_valid = min(BN, a.S - k0);
+            sk.load(kp + (int64_t)k0 * a.k.stride_s, a.k.stride_s, rows_valid, tid);
+            sv.load(vp + (int64_t)k0 * a.v.stride_s, a.v.stride_s, rows_valid, tid);
+            if (partial && drow && tid < BN) kd_next = drow[min(k0 + tid, a.S - 1)];
+        }
+
+        bool act[2];
 #pragma unroll
-            for (int nb = 0; nb < 2; ++nb) {
-                const int kb0 = k0 + 32 * nb;
-                bool on = kb0 < a.S;
-                if (partial && bounded && kb0 > qw_hi) on = false;
-                if (partial && a.window >= 0 && (int64_t)qw_lo - (kb0 + 31) > a.window) on = false;
-                act[nb] = on;
+        for (int nb = 0; nb < 2; ++nb) {
+            const int kb0 = ck0 + 32 * nb;
+            bool on = kb0 < a.S;
+            if (cpartial && bounded && kb0 > qw_hi) on = false;
+            if (cpartial && a.window >= 0 && (int64_t)qw_lo - (kb0 + 31) > a.window) on = false;
+            act[nb] = on;
+        }
+        if (!act[0] && !act[1]) continue;
+
+        // S^T blocks (kv x q)
+        f32x16 s[2];
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) s[nb][v] = 0.f;
+            if (act[nb]) {
+#pragma unroll
+                for (int kk = 0; kk < KK; ++kk) s[nb] = mfma32(TL::row_frag(Ks, rbase, 32 * nb, kk), qf[kk], s[nb]);
             }
-            if (!act[0] && !act[1]) continue;
-
-            // S^T blocks (kv x q), already in log2 units after the scale
-            f32x16 s[2];
-#pragma unroll
-            for (int nb = 0; nb < 2; ++nb) {
-#pragma unroll
-                for (int v = 0; v < 16; ++v) s[nb][v] = 0.f;
-                if (act[nb]) {
-#pragma unroll
-                    for (int kk = 0; kk < KK; ++kk)
-                        s[nb] = mfma32(row_frag<D>(Ks, 32 * nb + r, 2 * kk + hh), qf[kk], s[nb]);
-                }
-            }
-            float mx = -INFINITY;
+        }
+        // scale into log2 units and mask
+        float mx = -INFINITY;
+        if (cpartial) {
+            // d = q - kv for element v is qrel - (32*nb + 8*(v/4) + v%4); all tests are branch-free
+            const int qrel = q - ck0 - 4 * hh;
+            const int dmin = bounded ? 0 : -0x40000000;        // kv <= q
+            const int dend = q - a.S;                           // kv < S  <=>  d > q - S
 #pragma unroll
             for (int nb = 0; nb < 2; ++nb) {
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
-                    float x = s[nb][v] * sl2;
-                    bool ok = act[nb];
-                    if (partial) {
-                        const int kl = 32 * nb + 8 * (v >> 2) + 4 * hh + (v & 3);
-                        const int kv = k0 + kl;
-                        ok = ok && kv < a.S && pair_allowed(q, kv, a.causal, a.window);
-                        if (drow) ok = ok && (kdoc[kl] == docq);
-                    }
-                    x = ok ? x : -INFINITY;
+                    const int kc = 32 * nb + 8 * (v >> 2) + (v & 3);
+                    const int d = qrel - kc;
+                    bool ok = (d >= dmin) & (d <= wlim) & (d > dend) & act[nb];
+                    if (drow) ok = ok & (kdoc[kc + 4 * hh] == docq);
+                    const float x = ok ? s[nb][v] * sl2 : -INFINITY;
                     s[nb][v] = x;
                     mx = fmaxf(mx, x);
                 }
             }
-            mx = fmaxf(mx, xor32(mx));
-            const float mn = fmaxf(m, mx);
-            const float mu = mn == -INFINITY ? 0.f : mn;
-            const float alpha = fast_exp2(m - mu);
-            float rs = 0.f;
-            bf16x8 pf[2][2];
+        } else {
 #pragma unroll
             for (int nb = 0; nb < 2; ++nb) {
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
-                    const float p = fast_exp2(s[nb][v] - mu);
-                    rs += p;
-                    pf[nb][v >> 3][v & 7] = (__bf16)p;
+                    const float x = s[nb][v] * sl2;
+                    s[nb][v] = x;
+                    mx = fmaxf(mx, x);
                 }
             }
-            rs += xor32(rs);
-            lsum = lsum * alpha + rs;
-            m = mn;
+        }
+        mx = fmaxf(mx, xor32(mx));
+        // Lazy rescaling: the running reference m only moves when the row maximum has grown by more
+        // than kSlack (in log2 units), so exp2(x - m) stays below 2^kSlack and the accumulator
+        // rescale is a rare, wave-uniform branch instead of 128 multiplies per step.
+        constexpr float kSlack = 8.0f;
+        const bool grow = mx > m + kSlack;      // false while mx == -inf (nothing visible yet)
+        if (__any(grow)) {
+            const float mn = grow ? mx : m;
+            const float alpha = m == -INFINITY ? 0.f : fast_exp2(m - mn);
+            lsum *= alpha;
 #pragma unroll
             for (int db = 0; db < DB; ++db)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) o[db][v] *= alpha;
+            m = mn;
+        }
+        const float mu = m == -INFINITY ? 0.f : m;
+        float rs = 0.f;
+        bf16x8 pf[2][2];
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const float p = fast_exp2(s[nb][v] - mu);
+                rs += p;
+                pf[nb][v >> 3][v & 7] = (__bf16)p;
+            }
+        }
+        rs += xor32(rs);
+        lsum += rs;
 
-            // O^T += V^T P^T
+        // O^T += V^T P^T
 #pragma unroll
-            for (int nb = 0; nb < 2; ++nb) {
-                if (!act[nb]) continue;
+        for (int nb = 0; nb < 2; ++nb) {
+            if (!act[nb]) continue;
 #pragma unroll
-                for (int t = 0; t < 2; ++t) {
+            for (int t = 0; t < 2; ++t) {
 #pragma unroll
-                    for (int db = 0; db < DB; ++db)
-                        o[db] = mfma32(tr_frag<D>(Vs, 32 * nb + 16 * t, 32 * db, lane), pf[nb][t], o[db]);
-                }
+                for (int db = 0; db < DB; ++db)
+                    o[db] = mfma32(TL::tr_frag(Vs, tbase, 32 * nb + 16 * t, 32 * db), pf[nb][t], o[db]);
             }
         }
     }
@@ -183,13 +250,13 @@ __global__ __launch_bounds__(kFwdThreads) void attn_fwd_bf16_kernel(AttnArgs a) 
 
 template <int D>
 static int fwd_d(const AttnArgs& a, hipStream_t st) {
-    const size_t lds = (size_t)2 * kFwdBN * D * 2 + kFwdBN * 8;
+    const size_t lds = (size_t)2 * Tile<D>::bytes(kFwdBN) + kFwdBN * 8;
     if (lds > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_bf16_kernel<D>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return fail(MA_ERR_LAUNCH, "hipFuncSetAttribute(attn_fwd_bf16, %zu): %s", lds, hipGetErrorString(e));
     }
-    hipLaunchKernelGGL(attn_fwd_bf16_kernel<D>, dim3(a.T, a.Hq, a.B), dim3(kFwdThreads), lds, st, a);
+    hipLaunchKernelGGL(attn_fwd_bf16_kernel<D>, dim3(a.B * a.Hq, a.T, 1), dim3(kFwdThreads), lds, st, a);
     return check_launch("attn_fwd_bf16_kernel");
 }
 
