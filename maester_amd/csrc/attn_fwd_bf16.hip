@@ -21,6 +21,8 @@ namespace ma {
 constexpr int kFwdThreads = 256;
 constexpr int kFwdBN = 64;  // kv rows per step
 
+constexpr int kPipe = 4;  // LDS fragment reads kept in flight ahead of the MFMAs
+
 // Walks the (partial, then full) kv tile lists of one q tile in steps of BN rows, skipping the
 // steps no row of the workgroup can see.  All state is workgroup-uniform.
 struct KvSteps {
@@ -48,23 +50,48 @@ struct KvSteps {
     }
 };
 
-template <int D>
+// Workgroup id -> (q tile, q head, batch row).  Workgroups are handed to the 8 XCDs round-robin by
+// id, and each XCD has its own L2; when the (batch row, kv head) pairs divide evenly over the XCDs
+// every pair is pinned to one XCD, so the q heads and q tiles that stream the same K/V rows share
+// an L2.  Inside an XCD the late q tiles (most keys under causality) are started first.
+__device__ __forceinline__ void map_workgroup(const AttnArgs& a, int id, int& i, int& h, int& b) {
+    constexpr int kXcd = 8;
+    const int G = a.Hq / a.Hkv;
+    const int pairs = a.B * a.Hkv;
+    if (pairs % kXcd == 0) {
+        const int ppx = pairs / kXcd;  // pairs per XCD
+        const int xcd = id % kXcd, n = id / kXcd;
+        i = a.T - 1 - n / (ppx * G);
+        const int rem = n % (ppx * G);
+        const int pair = xcd * ppx + rem / G;
+        b = pair / a.Hkv;
+        h = (pair % a.Hkv) * G + rem % G;
+    } else {
+        i = a.T - 1 - id / (a.B * a.Hq);
+        const int rem = id % (a.B * a.Hq);
+        b = rem / a.Hq;
+        h = rem % a.Hq;
+    }
+}
+
+template <int D, bool HAS_DOC>
 __global__ __launch_bounds__(kFwdThreads) void attn_fwd_bf16_kernel(AttnArgs a) {
     using TL = Tile<D>;
     constexpr int KK = D / 16;  // contraction steps of S^T
     constexpr int DB = D / 32;  // 32-row blocks of O^T
     constexpr int BN = kFwdBN;
     extern __shared__ __align__(16) char smem_raw[];
-    lds_ptr Ks = (lds_ptr)smem_raw;
-    lds_ptr Vs = Ks + TL::bytes(BN);
-    MA_LDS int64_t* kdoc = (MA_LDS int64_t*)(Vs + TL::bytes(BN));
+    // double-buffered K and V tiles and kv document ids
+    const lds_ptr lds0 = (lds_ptr)smem_raw;
+    auto Kbuf = [&](int i) { return lds0 + i * 2 * TL::bytes(BN); };
+    auto Vbuf = [&](int i) { return lds0 + i * 2 * TL::bytes(BN) + TL::bytes(BN); };
+    auto Dbuf = [&](int i) { return (MA_LDS int64_t*)(lds0 + 4 * TL::bytes(BN)) + i * BN; };
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keep it in a scalar register
     const int r = lane & 31, hh = lane >> 5;
-    // x walks (batch row, head), y walks q tiles from the last (most keys under causality) to the first
-    const int i = gridDim.y - 1 - blockIdx.y;
-    const int h = blockIdx.x % a.Hq, b = blockIdx.x / a.Hq;
+    int i, h, b;
+    map_workgroup(a, blockIdx.x, i, h, b);
     const int hk = h / (a.Hq / a.Hkv);
     const int qw_lo = i * kTile + 32 * w, qw_hi = qw_lo + 31;
     const int q = qw_lo + r;
@@ -74,14 +101,11 @@ __global__ __launch_bounds__(kFwdThreads) void attn_fwd_bf16_kernel(AttnArgs a) 
     const __bf16* qp = (const __bf16*)a.q.ptr + b * a.q.stride_b + h * a.q.stride_h;
     const __bf16* kp = (const __bf16*)a.k.ptr + b * a.k.stride_b + hk * a.k.stride_h;
     const __bf16* vp = (const __bf16*)a.v.ptr + b * a.v.stride_b + hk * a.v.stride_h;
-    const int64_t* drow = a.doc ? a.doc + (size_t)b * a.S : nullptr;
+    const int64_t* drow = HAS_DOC ? a.doc + (size_t)b * a.S : nullptr;
 
     // rows past the end of the sequence read the last valid row; their results are never stored
     const int qc = min(q, a.S - 1);
-    bf16x8 qf[KK];
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk) qf[kk] = *(const bf16x8*)(qp + (int64_t)qc * a.q.stride_s + 16 * kk + 8 * hh);
-    const int64_t docq = drow ? drow[qc] : 0;
+    const int64_t docq = HAS_DOC ? drow[qc] : 0;
     const int wlim = a.window >= 0 ? (int)min(a.window, (int64_t)0x3fffffff) : 0x7fffffff;
 
     f32x16 o[DB];
@@ -102,24 +126,41 @@ __global__ __launch_bounds__(kFwdThreads) void attn_fwd_bf16_kernel(AttnArgs a) 
     st.it = 0; st.half = -1; st.S = a.S; st.q_lo = i * kTile; st.q_hi = i * kTile + kTile - 1;
     st.bounded = bounded; st.window = a.window;
 
-    Stager<D, BN, kFwdThreads> sk, sv;
+    DirectStager<D, BN, kFwdThreads / 64> sk, sv;
+    sk.init(w, lane, a.k.stride_s);
+    sv.init(w, lane, a.v.stride_s);
     int64_t kd_next = 0;
     bool have = st.next();
-    int k0 = st.k0, rows_valid = 0;
+    int k0 = st.k0;
     bool partial = st.partial;
     if (have) {
-        rows_valid = min(BN, a.S - k0);
-        sk.load(kp + (int64_t)k0 * a.k.stride_s, a.k.stride_s, rows_valid, tid);
-        sv.load(vp + (int64_t)k0 * a.v.stride_s, a.v.stride_s, rows_valid, tid);
-        if (partial && drow && tid < BN) kd_next = drow[min(k0 + tid, a.S - 1)];
+        const int rows_valid = min(BN, a.S - k0);
+        sk.issue(kp + (int64_t)k0 * a.k.stride_s, Kbuf(0), w, lane, rows_valid, a.k.stride_s);
+        sv.issue(vp + (int64_t)k0 * a.v.stride_s, Vbuf(0), w, lane, rows_valid, a.v.stride_s);
+        if (HAS_DOC && partial && tid < BN) kd_next = drow[min(k0 + tid, a.S - 1)];
+    }
+    // The Q tile comes in through LDS too (coalesced 1 KB runs instead of 32 strided rows per
+    // load); it borrows the second K/V buffer pair, which the first step does not use yet.
+    bf16x8 qf[KK];
+    {
+        lds_ptr Qs = Kbuf(1);
+        DirectStager<D, kTile, kFwdThreads / 64> sq;
+        sq.init(w, lane, a.q.stride_s);
+        sq.issue(qp + (int64_t)i * kTile * a.q.stride_s, Qs, w, lane, min(kTile, a.S - i * kTile), a.q.stride_s);
+        wait_vmem();
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) qf[kk] = TL::row_frag(Qs, rbase, 32 * w, kk);
+        __syncthreads();  // all Q fragments are in registers before the buffers are reused
     }
 
-    while (have) {
-        __syncthreads();  // everyone is done reading the previous tiles
-        sk.store(Ks, rows_valid, tid);
-        sv.store(Vs, rows_valid, tid);
-        if (partial && drow && tid < BN) kdoc[tid] = kd_next;
-        __syncthreads();
+    for (int n = 0; have; ++n) {
+        const int cur = n & 1;
+        lds_ptr Ks = Kbuf(cur), Vs = Vbuf(cur);
+        MA_LDS int64_t* kdoc = Dbuf(cur);
+        if (HAS_DOC && partial && tid < BN) kdoc[tid] = kd_next;
+        wait_vmem();       // this wave's share of the current tiles has landed ...
+        __syncthreads();   // ... and so has everyone's; all waves are also done with the other buffers
 
         const int ck0 = k0;
         const bool cpartial = partial;
@@ -127,10 +168,10 @@ __global__ __launch_bounds__(kFwdThreads) void attn_fwd_bf16_kernel(AttnArgs a) 
         if (have) {
             k0 = st.k0;
             partial = st.partial;
-            rows_valid = min(BN, a.S - k0);
-            sk.load(kp + (int64_t)k0 * a.k.stride_s, a.k.stride_s, rows_valid, tid);
-            sv.load(vp + (int64_t)k0 * a.v.stride_s, a.v.stride_s, rows_valid, tid);
-            if (partial && drow && tid < BN) kd_next = drow[min(k0 + tid, a.S - 1)];
+            const int rows_valid = min(BN, a.S - k0);
+            sk.issue(kp + (int64_t)k0 * a.k.stride_s, Kbuf(cur ^ 1), w, lane, rows_valid, a.k.stride_s);
+            sv.issue(vp + (int64_t)k0 * a.v.stride_s, Vbuf(cur ^ 1), w, lane, rows_valid, a.v.stride_s);
+            if (HAS_DOC && partial && tid < BN) kd_next = drow[min(k0 + tid, a.S - 1)];
         }
 
         bool act[2];
@@ -144,36 +185,46 @@ __global__ __launch_bounds__(kFwdThreads) void attn_fwd_bf16_kernel(AttnArgs a) 
         }
         if (!act[0] && !act[1]) continue;
 
-        // S^T blocks (kv x q)
+        // S^T blocks (kv x q).  Both 32-row blocks are always computed: a block the wave cannot see
+        // is masked below, and keeping one straight-line path keeps every accumulator in place.
         f32x16 s[2];
-#pragma unroll
-        for (int nb = 0; nb < 2; ++nb) {
-#pragma unroll
-            for (int v = 0; v < 16; ++v) s[nb][v] = 0.f;
-            if (act[nb]) {
-#pragma unroll
-                for (int kk = 0; kk < KK; ++kk) s[nb] = mfma32(TL::row_frag(Ks, rbase, 32 * nb, kk), qf[kk], s[nb]);
-            }
-        }
+        rowfrag_gemm<D, 2, kPipe>(lds_addr(Ks) + rbase, qf, s);
         // scale into log2 units and mask
         float mx = -INFINITY;
         if (cpartial) {
-            // d = q - kv for element v is qrel - (32*nb + 8*(v/4) + v%4); all tests are branch-free
+            // d = q - kv for element v is qrel - (32*nb + 8*(v/4) + v%4).  The causal, window and
+            // end-of-sequence tests together are one range test dlo <= d <= dhi, done as a single
+            // unsigned compare of (d - dlo) against (dhi - dlo).
             const int qrel = q - ck0 - 4 * hh;
-            const int dmin = bounded ? 0 : -0x40000000;        // kv <= q
-            const int dend = q - a.S;                           // kv < S  <=>  d > q - S
+            const int dlo = max(bounded ? 0 : -0x40000000, q - a.S + 1);   // kv <= q, kv < S
+            const unsigned span = (unsigned)(wlim - dlo);                   // wlim >= dlo is not required:
+            const bool some = wlim >= dlo;                                  // an empty range hides everything
+            const unsigned t0 = (unsigned)(qrel - dlo);
 #pragma unroll
             for (int nb = 0; nb < 2; ++nb) {
+                // ids of the 16 kv rows of this block the lane owns: 4 groups of 4 consecutive rows
+                i64x2 ids[4][2];
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const int kc = 32 * nb + 8 * (v >> 2) + (v & 3);
-                    const int d = qrel - kc;
-                    bool ok = (d >= dmin) & (d <= wlim) & (d > dend) & act[nb];
-                    if (drow) ok = ok & (kdoc[kc + 4 * hh] == docq);
-                    const float x = ok ? s[nb][v] * sl2 : -INFINITY;
-                    s[nb][v] = x;
-                    mx = fmaxf(mx, x);
+                for (int g = 0; g < 4; ++g) {
+                    ids[g][0] = ids[g][1] = i64x2{0, 0};
+                    if (HAS_DOC) {
+                        ids[g][0] = *(MA_LDS i64x2*)(kdoc + 32 * nb + 8 * g + 4 * hh);
+                        ids[g][1] = *(MA_LDS i64x2*)(kdoc + 32 * nb + 8 * g + 4 * hh + 2);
+                    }
                 }
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int v = 4 * g + e;
+                        bool ok = (t0 - (unsigned)(32 * nb + 8 * g + e) <= span) & some & act[nb];
+                        if (HAS_DOC) ok = ok & (ids[g][e >> 1][e & 1] == docq);
+                        const float x = ok ? s[nb][v] * sl2 : -INFINITY;
+                        s[nb][v] = x;
+                        mx = fmaxf(mx, x);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);  // finish this block before starting the next
             }
         } else {
 #pragma unroll
@@ -218,21 +269,17 @@ __global__ __launch_bounds__(kFwdThreads) void attn_fwd_bf16_kernel(AttnArgs a) 
         lsum += rs;
 
         // O^T += V^T P^T
-#pragma unroll
-        for (int nb = 0; nb < 2; ++nb) {
-            if (!act[nb]) continue;
-#pragma unroll
-            for (int t = 0; t < 2; ++t) {
-#pragma unroll
-                for (int db = 0; db < DB; ++db)
-                    o[db] = mfma32(TL::tr_frag(Vs, tbase, 32 * nb + 16 * t, 32 * db), pf[nb][t], o[db]);
-            }
-        }
+        trfrag_gemm<D, 4, kPipe>(lds_addr(Vs) + tbase, &pf[0][0], o);
     }
 
-    if (qvalid) {
+    // Epilogue: O^T (a lane owns one q row, 4 consecutive d per register group) goes through LDS so
+    // that the global stores are whole 16-byte-per-lane row segments.
+    __syncthreads();  // every wave is done with the K/V buffers
+    mfma_fence();
+    {
+        constexpr int kPitchO = D * 2 + 16;
+        lds_ptr Os = lds0 + w * 32 * kPitchO;
         const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
-        __bf16* op = (__bf16*)a.o.ptr + b * a.o.stride_b + (int64_t)q * a.o.stride_s + h * a.o.stride_h;
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
 #pragma unroll
@@ -240,24 +287,38 @@ __global__ __launch_bounds__(kFwdThreads) void attn_fwd_bf16_kernel(AttnArgs a) 
                 bf16x4 pk;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) pk[e] = (__bf16)(o[db][4 * g + e] * inv);
-                *(bf16x4*)(op + 32 * db + 8 * g + 4 * hh) = pk;
+                *(MA_LDS bf16x4*)(Os + r * kPitchO + (32 * db + 8 * g + 4 * hh) * 2) = pk;
             }
         }
-        if (hh == 0)
+        constexpr int CH = D / 8, RPI = 64 / CH;  // rows per store instruction
+        const int rsub = lane / CH, c = lane % CH;
+        __bf16* ob = (__bf16*)a.o.ptr + b * a.o.stride_b + h * a.o.stride_h;
+#pragma unroll
+        for (int it = 0; it < 32 / RPI; ++it) {
+            const int row = it * RPI + rsub;
+            const u32x4 val = *(MA_LDS u32x4*)(Os + row * kPitchO + c * 16);
+            if (qw_lo + row < a.S) *(u32x4*)(ob + (int64_t)(qw_lo + row) * a.o.stride_s + c * 8) = val;
+        }
+        if (qvalid && hh == 0)
             a.lse[((size_t)b * a.Hq + h) * a.S + q] = lsum > 0.f ? (m + __log2f(lsum)) * kLn2 : -INFINITY;
     }
 }
 
-template <int D>
-static int fwd_d(const AttnArgs& a, hipStream_t st) {
-    const size_t lds = (size_t)2 * Tile<D>::bytes(kFwdBN) + kFwdBN * 8;
+template <int D, bool HAS_DOC>
+static int fwd_dd(const AttnArgs& a, hipStream_t st) {
+    const size_t lds = (size_t)4 * Tile<D>::bytes(kFwdBN) + 2 * kFwdBN * 8;
     if (lds > 64 * 1024) {
-        hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_bf16_kernel<D>,
+        hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_bf16_kernel<D, HAS_DOC>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return fail(MA_ERR_LAUNCH, "hipFuncSetAttribute(attn_fwd_bf16, %zu): %s", lds, hipGetErrorString(e));
     }
-    hipLaunchKernelGGL(attn_fwd_bf16_kernel<D>, dim3(a.B * a.Hq, a.T, 1), dim3(kFwdThreads), lds, st, a);
+    hipLaunchKernelGGL((attn_fwd_bf16_kernel<D, HAS_DOC>), dim3(a.B * a.Hq * a.T, 1, 1), dim3(kFwdThreads), lds, st, a);
     return check_launch("attn_fwd_bf16_kernel");
+}
+
+template <int D>
+static int fwd_d(const AttnArgs& a, hipStream_t st) {
+    return a.doc ? fwd_dd<D, true>(a, st) : fwd_dd<D, false>(a, st);
 }
 
 int launch_attn_fwd_bf16(const AttnArgs& a, hipStream_t st) {

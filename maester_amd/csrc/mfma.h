@@ -20,6 +20,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
 
 namespace ma {
 
@@ -28,9 +29,19 @@ typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef int64_t i64x2 __attribute__((ext_vector_type(2)));
 
 #define MA_LDS __attribute__((address_space(3)))
 typedef MA_LDS char* lds_ptr;
+
+// compile-time loop: f(std::integral_constant<int, I>{}) for I in [B, E)
+template <int B, int E, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (B < E) {
+        f(std::integral_constant<int, B>{});
+        static_for<B + 1, E>(f);
+    }
+}
 
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
@@ -83,6 +94,132 @@ __device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
 }
 
+// MFMAs with the register classes of their operands pinned.  Left to itself the register
+// allocator keeps long-lived accumulators in AGPRs and shuttles all of them to VGPRs and back
+// around every loop iteration as soon as anything (a rare rescale, say) touches them with the
+// vector ALU.  Here the accumulators are pinned to VGPRs ("+v": MFMA reads/writes them in place
+// and so does the VALU) and the loop-invariant operand fragments can be parked in AGPRs ("a").
+// The compiler does not know these asm statements are MFMAs and pads no hazards: callers keep
+// VALU readers of c at least 16 wait states behind the last MFMA (mfma_fence()) and VALU writers
+// of a/b a few instructions ahead of the first.
+__device__ __forceinline__ void mfma32_vv(f32x16& c, bf16x8 a, bf16x8 b) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void mfma32_va(f32x16& c, bf16x8 a, bf16x8 b_agpr) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b_agpr));
+}
+__device__ __forceinline__ void mfma32_av(f32x16& c, bf16x8 a_agpr, bf16x8 b) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "a"(a_agpr), "v"(b));
+}
+// same with a zero addend: starts an accumulation without a VALU-written zero tile
+__device__ __forceinline__ void mfma32_va_zero(f32x16& c, bf16x8 a, bf16x8 b_agpr) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "a"(b_agpr));
+}
+__device__ __forceinline__ void mfma32_av_zero(f32x16& c, bf16x8 a_agpr, bf16x8 b) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "a"(a_agpr), "v"(b));
+}
+__device__ __forceinline__ void mfma32_vv_zero(f32x16& c, bf16x8 a, bf16x8 b) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
+}
+// 16 wait states: enough for the result of an 8-pass MFMA to be readable by the vector ALU
+__device__ __forceinline__ void mfma_fence() { asm volatile("s_nop 15"); }
+
+// ---- explicitly pipelined LDS fragment reads ---------------------------------------------------
+// The compiler serialises "LDS read -> wait -> MFMA" in these kernels, so the hot loops issue
+// their LDS reads through asm statements (kept in program order) and tie the matching
+// s_waitcnt to the fragment it guards: lds_wait<N>(x) returns once at most N younger LDS
+// operations are still outstanding, and because it takes x as a read-write operand no consumer
+// of x can be moved above it.  Extra outstanding operations the compiler adds only make the
+// waits more conservative.  The MFMAs stay builtins, so the compiler keeps handling their hazards.
+template <int OFF>
+__device__ __forceinline__ bf16x8 lds_read_b128(uint32_t addr) {
+    bf16x8 v;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
+    return v;
+}
+template <int OFF>
+__device__ __forceinline__ bf16x4 lds_read_tr16_b64(uint32_t addr) {
+    bf16x4 v;
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
+    return v;
+}
+template <int N>
+__device__ __forceinline__ void lds_wait(bf16x8& x) {
+    asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(x) : "n"(N));
+}
+__device__ __forceinline__ uint32_t lds_addr(lds_ptr p) { return (uint32_t)(uintptr_t)p; }
+
+// acc[nb] = sum_kk L(rows 32nb + r, cols 16kk..) x reg[kk] for NB row blocks of 32 at once: a
+// software pipeline of depth P over the NB*KK row-wise fragments of an LDS tile (row_addr = lds
+// address of the tile + Tile::row_base(lane)).  The register-resident fragments reg[] live in
+// AGPRs.  SWAP puts the LDS fragment in the B slot instead (computes the transposed product).
+// acc is overwritten (no zero tile needed) and lives in VGPRs; ends with mfma_fence().
+template <int D, int NB, int P, bool SWAP = false>
+__device__ __forceinline__ void rowfrag_gemm(uint32_t row_addr, const bf16x8* reg, f32x16* acc) {
+    using TL = Tile<D>;
+    constexpr int KK = D / 16;
+    constexpr int N = NB * KK;
+    bf16x8 t[N];
+    auto rd = [&](auto idx) {
+        constexpr int i = decltype(idx)::value;
+        constexpr int kk = i / NB, nb = i % NB;
+        t[i] = lds_read_b128<nb * 32 * TL::kPitch + kk * 32>(row_addr);
+    };
+    auto step = [&](auto idx) {
+        constexpr int i = decltype(idx)::value;
+        constexpr int kk = i / NB, nb = i % NB;
+        constexpr int younger = (N - 1 - i) < (P - 1) ? (N - 1 - i) : (P - 1);
+        lds_wait<younger>(t[i]);
+        if constexpr (kk == 0) {
+            if constexpr (SWAP) mfma32_av_zero(acc[nb], reg[kk], t[i]);
+            else mfma32_va_zero(acc[nb], t[i], reg[kk]);
+        } else {
+            if constexpr (SWAP) mfma32_av(acc[nb], reg[kk], t[i]);
+            else mfma32_va(acc[nb], t[i], reg[kk]);
+        }
+    };
+    static_for<0, (P < N ? P : N)>(rd);
+    static_for<0, N>([&](auto idx) {
+        constexpr int i = decltype(idx)::value;
+        step(idx);
+        if constexpr (i + P < N) rd(std::integral_constant<int, i + P>{});
+    });
+    mfma_fence();
+}
+
+// acc[db] += L^T(rows 16j.., cols 32db..) x reg[j] over NJ 16-row slabs of an LDS tile through
+// transposed fragments (tr_addr = lds address of the tile + Tile::tr_base(lane)).  Pipeline of
+// depth P over the NJ * DB fragments (two LDS reads each).  acc and reg live in VGPRs; ends with
+// mfma_fence().
+template <int D, int NJ, int P>
+__device__ __forceinline__ void trfrag_gemm(uint32_t tr_addr, const bf16x8* reg, f32x16* acc) {
+    using TL = Tile<D>;
+    constexpr int DB = D / 32;
+    constexpr int N = NJ * DB;
+    bf16x4 lo[N], hi[N];
+    auto rd = [&](auto idx) {
+        constexpr int i = decltype(idx)::value;
+        constexpr int j = i / DB, db = i % DB;
+        lo[i] = lds_read_tr16_b64<(16 * j) * TL::kPitch + db * 64>(tr_addr);
+        hi[i] = lds_read_tr16_b64<(16 * j + 2) * TL::kPitch + db * 64>(tr_addr);
+    };
+    auto step = [&](auto idx) {
+        constexpr int i = decltype(idx)::value;
+        constexpr int j = i / DB, db = i % DB;
+        constexpr int younger = (N - 1 - i) < (P - 1) ? (N - 1 - i) : (P - 1);
+        bf16x8 f = __builtin_shufflevector(lo[i], hi[i], 0, 1, 2, 3, 4, 5, 6, 7);
+        lds_wait<2 * younger>(f);
+        mfma32_vv(acc[db], f, reg[j]);
+    };
+    static_for<0, (P < N ? P : N)>(rd);
+    static_for<0, N>([&](auto idx) {
+        constexpr int i = decltype(idx)::value;
+        step(idx);
+        if constexpr (i + P < N) rd(std::integral_constant<int, i + P>{});
+    });
+    mfma_fence();  // whatever the compiler schedules next may read acc with the vector ALU
+}
+
 // Global -> registers -> LDS staging of a ROWS x D bf16 tile by NT threads.  load() issues all the
 // global loads of the thread back to back (rows past the end are clamped to the last valid row so
 // that the loads need no branches; their data is zeroed in store()), store() writes them to LDS.
@@ -114,6 +251,60 @@ struct Stager {
         for (int n = 0; n < N; ++n) *(MA_LDS u32x4*)(tile + Tile<D>::off(r0 + n * RPP, c * 8)) = v[n];
     }
 };
+
+// Global -> LDS staging without registers (gfx950 global_load_lds_dwordx4): every lane of a wave
+// moves 16 bytes from an address of its own to LDS at wave_base + 16*lane, asynchronously (counted
+// by vmcnt).  The tile is cut into runs of 64 consecutive 16-byte slots (the pad slot of each row
+// included; it receives a copy of chunk 0); run t is moved by wave t % NWAVES.  Which global
+// (row, chunk) lands in a slot is decided on the global side, so the permuted/padded layout costs
+// nothing.  Rows at or beyond rows_valid re-read the last valid row (callers mask them).
+#define MA_GLB __attribute__((address_space(1)))
+template <int D, int ROWS, int NWAVES>
+struct DirectStager {
+    using TL = Tile<D>;
+    static constexpr int SPR = TL::kChunks + 1;  // slots per row
+    static constexpr int SLOTS = ROWS * SPR;
+    static_assert(SLOTS % 64 == 0, "tile must be a whole number of wave runs");
+    static constexpr int NL = SLOTS / 64;
+    static constexpr int PER = (NL + NWAVES - 1) / NWAVES;
+    uint32_t off[PER];  // byte offset of this lane's source from the first row of the tile
+
+    __device__ __forceinline__ static void slot(int t, int lane, int& row, int& chunk) {
+        const int s = t * 64 + lane;
+        const int rho = s / SPR;
+        chunk = s - rho * SPR;
+        if (chunk == TL::kChunks) chunk = 0;
+        row = TL::prow(rho);  // prow is its own inverse
+    }
+    __device__ __forceinline__ void init(int w, int lane, int64_t stride) {
+#pragma unroll
+        for (int p = 0; p < PER; ++p) {
+            int row, chunk;
+            slot(w + p * NWAVES, lane, row, chunk);
+            off[p] = (uint32_t)((row * stride + chunk * 8) * 2);
+        }
+    }
+    __device__ __forceinline__ void issue(const __bf16* g, lds_ptr tile, int w, int lane, int rows_valid,
+                                          int64_t stride) const {
+#pragma unroll
+        for (int p = 0; p < PER; ++p) {
+            const int t = w + p * NWAVES;
+            if (t < NL) {
+                uint32_t o = off[p];
+                if (rows_valid < ROWS) {
+                    int row, chunk;
+                    slot(t, lane, row, chunk);
+                    o = (uint32_t)((min(row, rows_valid - 1) * stride + chunk * 8) * 2);
+                }
+                __builtin_amdgcn_global_load_lds((const MA_GLB void*)((const char*)g + o), (MA_LDS void*)(tile + t * 1024),
+                                                 16, 0, 0);
+            }
+        }
+    }
+};
+
+// waits until this wave's outstanding global (and global->LDS) loads have landed
+__device__ __forceinline__ void wait_vmem() { __builtin_amdgcn_s_waitcnt(0x0f70); }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
