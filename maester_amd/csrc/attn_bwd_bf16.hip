@@ -20,7 +20,64 @@
 namespace ma {
 
 constexpr int kBwdThreads = 256;
-constexpr int kStep = 64;  // rows staged per step
+constexpr int kStep = 64;   // rows staged per step
+constexpr int kBPipe = 4;   // LDS fragment reads kept in flight ahead of the MFMAs
+constexpr int kXcd = 8;
+
+// Workgroup id -> (tile, head, batch row) with every (batch row, kv head) pair pinned to one XCD
+// (workgroups go to the XCDs round-robin by id; each XCD has its own L2) when the pairs divide
+// evenly.  `heads` is the number of heads per kv head the grid enumerates (G for q-head grids, 1
+// for kv-head grids); `first_heavy` says whether tile 0 (true) or tile T-1 (false) is the
+// longest-running one, which is started first.
+__device__ __forceinline__ void map_workgroup_bwd(const AttnArgs& a, int id, int heads, bool first_heavy, int& tile,
+                                                  int& head, int& b) {
+    const int pairs = a.B * a.Hkv;
+    int t;
+    if (pairs % kXcd == 0) {
+        const int ppx = pairs / kXcd;
+        const int xcd = id % kXcd, n = id / kXcd;
+        t = n / (ppx * heads);
+        const int rem = n % (ppx * heads);
+        const int pair = xcd * ppx + rem / heads;
+        b = pair / a.Hkv;
+        head = (pair % a.Hkv) * heads + rem % heads;
+    } else {
+        t = id / (a.B * a.Hkv * heads);
+        const int rem = id % (a.B * a.Hkv * heads);
+        b = rem / (a.Hkv * heads);
+        head = rem % (a.Hkv * heads);
+    }
+    tile = first_heavy ? t : a.T - 1 - t;
+}
+
+// O tile epilogue shared by the kernels: a wave holds a 32-row x D fp32 tile transposed in registers
+// (lane (r, hh) owns row r and, per 32-column block, columns 8g + 4hh + e); it is scaled, cast to
+// bf16, laid out row-major in the wave's LDS scratch and written out as 16-byte row segments.
+template <int D>
+__device__ __forceinline__ void store_tile_T(lds_ptr scratch, const f32x16* acc, float mul, __bf16* gbase, int64_t stride,
+                                            int row0, int rows_end, int lane) {
+    constexpr int DB = D / 32;
+    constexpr int kPitchO = D * 2 + 16;
+    const int r = lane & 31, hh = lane >> 5;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            bf16x4 pk;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) pk[e] = (__bf16)(acc[db][4 * g + e] * mul);
+            *(MA_LDS bf16x4*)(scratch + r * kPitchO + (32 * db + 8 * g + 4 * hh) * 2) = pk;
+        }
+    }
+    constexpr int CH = D / 8, RPI = 64 / CH;
+    const int rsub = lane / CH, c = lane % CH;
+#pragma unroll
+    for (int it = 0; it < 32 / RPI; ++it) {
+        const int row = it * RPI + rsub;
+        const u32x4 val = *(MA_LDS u32x4*)(scratch + row * kPitchO + c * 16);
+        if (row0 + row < rows_end) *(u32x4*)(gbase + (int64_t)(row0 + row) * stride + c * 8) = val;
+    }
+}
 
 // ------------------------------------------------------------------------------------------------
 // delta[b,h,q] = sum_d O[b,q,h,d] * dO[b,q,h,d]
@@ -51,23 +108,58 @@ __global__ __launch_bounds__(256) void attn_delta_bf16_kernel(AttnArgs a) {
 // ------------------------------------------------------------------------------------------------
 // dK / dV
 // ------------------------------------------------------------------------------------------------
-template <int D>
+// Walks, for each of the G query heads of the kv head, the (partial, then full) q tile lists of one
+// kv tile in steps of kStep q rows, skipping steps no row of the workgroup can see.
+struct QSteps {
+    const int32_t *plist, *flist;
+    int np, nf, G, g, it, half, S, k_lo, k_hi, bounded;
+    int64_t window;
+    int q0;
+    bool partial;
+
+    __device__ __forceinline__ bool next() {
+        for (;;) {
+            if (++half == kTile / kStep) {
+                half = 0;
+                if (++it >= np + nf) {
+                    it = 0;
+                    ++g;
+                }
+            }
+            if (g >= G || np + nf == 0) return false;
+            partial = it < np;
+            const int i = partial ? plist[it] : flist[it - np];
+            q0 = i * kTile + half * kStep;
+            if (q0 >= S) continue;
+            if (partial && bounded && q0 + kStep - 1 < k_lo) continue;
+            if (partial && window >= 0 && (int64_t)q0 - k_hi > window) continue;
+            return true;
+        }
+    }
+};
+
+template <int D, bool HAS_DOC>
 __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dkv_bf16_kernel(AttnArgs a) {
     using TL = Tile<D>;
     constexpr int KK = D / 16;
     constexpr int DB = D / 32;
     constexpr int BM = kStep;
+    constexpr int NW = kBwdThreads / 64;
     extern __shared__ __align__(16) char smem_raw[];
-    lds_ptr Qs = (lds_ptr)smem_raw;
-    lds_ptr Gs = Qs + TL::bytes(BM);  // dO rows
-    MA_LDS float* lse2s = (MA_LDS float*)(Gs + TL::bytes(BM));
-    MA_LDS float* dls = lse2s + BM;
-    MA_LDS int64_t* qdoc = (MA_LDS int64_t*)(dls + BM);
+    const lds_ptr lds0 = (lds_ptr)smem_raw;
+    // ring of two (Q, dO) tile pairs, then per-row lse / delta / document id for the two steps
+    auto Qbuf = [&](int i) { return lds0 + i * 2 * TL::bytes(BM); };
+    auto Gbuf = [&](int i) { return lds0 + i * 2 * TL::bytes(BM) + TL::bytes(BM); };
+    const lds_ptr aux = lds0 + 4 * TL::bytes(BM);
+    auto Lbuf = [&](int i) { return (MA_LDS float*)(aux) + i * BM; };
+    auto Ebuf = [&](int i) { return (MA_LDS float*)(aux + 2 * BM * 4) + i * BM; };
+    auto Dbuf = [&](int i) { return (MA_LDS int64_t*)(aux + 4 * BM * 4) + i * BM; };
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 31, hh = lane >> 5;
-    const int j = blockIdx.y, hk = blockIdx.x % a.Hkv, b = blockIdx.x / a.Hkv;
+    int j, hk, b;
+    map_workgroup_bwd(a, blockIdx.x, 1, true, j, hk, b);
     const int rbase = TL::row_base(lane), tbase = TL::tr_base(lane);
     const int G = a.Hq / a.Hkv;
     const int kw_lo = j * kTile + 32 * w, kw_hi = kw_lo + 31;
@@ -78,18 +170,29 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dkv_bf16_kernel(AttnArgs
 
     const __bf16* kp = (const __bf16*)a.k.ptr + b * a.k.stride_b + hk * a.k.stride_h;
     const __bf16* vp = (const __bf16*)a.v.ptr + b * a.v.stride_b + hk * a.v.stride_h;
-    const int64_t* drow = a.doc ? a.doc + (size_t)b * a.S : nullptr;
-
-    // rows past the end of the sequence read the last valid row; their results are masked / not stored
+    const int64_t* drow = HAS_DOC ? a.doc + (size_t)b * a.S : nullptr;
     const int kvc = min(kv, a.S - 1);
-    bf16x8 kf[KK], vf[KK];
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-        kf[kk] = *(const bf16x8*)(kp + (int64_t)kvc * a.k.stride_s + 16 * kk + 8 * hh);
-        vf[kk] = *(const bf16x8*)(vp + (int64_t)kvc * a.v.stride_s + 16 * kk + 8 * hh);
-    }
-    const int64_t dock = drow ? drow[kvc] : 0;
+    const int64_t dock = HAS_DOC ? drow[kvc] : 0;
     const int wlim = a.window >= 0 ? (int)min(a.window, (int64_t)0x3fffffff) : 0x7fffffff;
+
+    // K and V rows of the workgroup come in through LDS (coalesced) and stay in registers
+    bf16x8 kf[KK], vf[KK];
+    {
+        DirectStager<D, kTile, NW> sk, sv;
+        sk.init(w, lane, a.k.stride_s);
+        sv.init(w, lane, a.v.stride_s);
+        const int rows_valid = min(kTile, a.S - j * kTile);
+        sk.issue(kp + (int64_t)j * kTile * a.k.stride_s, Qbuf(0), w, lane, rows_valid, a.k.stride_s);
+        sv.issue(vp + (int64_t)j * kTile * a.v.stride_s, Qbuf(1), w, lane, rows_valid, a.v.stride_s);
+        wait_vmem();
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+            kf[kk] = TL::row_frag(Qbuf(0), rbase, 32 * w, kk);
+            vf[kk] = TL::row_frag(Qbuf(1), rbase, 32 * w, kk);
+        }
+        __syncthreads();
+    }
 
     f32x16 dkacc[DB], dvacc[DB];
 #pragma unroll
@@ -98,129 +201,172 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dkv_bf16_kernel(AttnArgs
         for (int v = 0; v < 16; ++v) dkacc[db][v] = dvacc[db][v] = 0.f;
 
     const size_t mrow = (size_t)b * a.T + j;
-    const int32_t* plist = a.map.q_indices + mrow * a.T;
-    const int32_t* flist = a.map.full_q_indices + mrow * a.T;
-    const int np = a.map.q_num_blocks[mrow];
-    const int nf = a.map.full_q_num_blocks[mrow];
+    QSteps st;
+    st.plist = a.map.q_indices + mrow * a.T;
+    st.flist = a.map.full_q_indices + mrow * a.T;
+    st.np = a.map.q_num_blocks[mrow];
+    st.nf = a.map.full_q_num_blocks[mrow];
+    st.G = G; st.g = 0; st.it = 0; st.half = -1; st.S = a.S;
+    st.k_lo = j * kTile; st.k_hi = j * kTile + kTile - 1; st.bounded = bounded; st.window = a.window;
 
-    for (int g = 0; g < G; ++g) {
-        const int h = hk * G + g;
-        const __bf16* qp = (const __bf16*)a.q.ptr + b * a.q.stride_b + h * a.q.stride_h;
-        const __bf16* gp = (const __bf16*)a.dout.ptr + b * a.dout.stride_b + h * a.dout.stride_h;
-        const size_t rowbase = ((size_t)b * a.Hq + h) * a.S;
-        for (int it = 0; it < np + nf; ++it) {
-            const bool partial = it < np;
-            const int i = partial ? plist[it] : flist[it - np];
-            for (int half = 0; half < kTile / BM; ++half) {
-                const int q0 = i * kTile + half * BM;
-                if (q0 >= a.S) continue;
-                if (partial && bounded && q0 + BM - 1 < j * kTile) continue;
-                if (partial && a.window >= 0 && (int64_t)q0 - (j * kTile + kTile - 1) > a.window) continue;
+    DirectStager<D, BM, NW> sq, sg;
+    sq.init(w, lane, a.q.stride_s);
+    sg.init(w, lane, a.dout.stride_s);
+    float lse_next = 0.f, dl_next = 0.f;
+    int64_t qd_next = 0;
+    auto issue = [&](int buf) {
+        const int h = hk * G + st.g;
+        const int q0 = st.q0;
+        const int rows_valid = min(BM, a.S - q0);
+        const __bf16* qp = (const __bf16*)a.q.ptr + b * a.q.stride_b + h * a.q.stride_h + (int64_t)q0 * a.q.stride_s;
+        const __bf16* gp = (const __bf16*)a.dout.ptr + b * a.dout.stride_b + h * a.dout.stride_h + (int64_t)q0 * a.dout.stride_s;
+        sq.issue(qp, Qbuf(buf), w, lane, rows_valid, a.q.stride_s);
+        sg.issue(gp, Gbuf(buf), w, lane, rows_valid, a.dout.stride_s);
+        if (tid < BM) {
+            const int qq = min(q0 + tid, a.S - 1);
+            const size_t row = ((size_t)b * a.Hq + h) * a.S + qq;
+            lse_next = a.lse[row] * kLog2e;
+            dl_next = a.delta[row];
+            if (HAS_DOC) qd_next = drow[qq];
+        }
+    };
+    bool have = st.next();
+    int q0 = st.q0;
+    bool partial = st.partial;
+    if (have) issue(0);
 
-                __syncthreads();
-                const int rows_valid = min(BM, a.S - q0);
-                {
-                    Stager<D, BM, kBwdThreads> sq, sg;
-                    sq.load(qp + (int64_t)q0 * a.q.stride_s, a.q.stride_s, rows_valid, tid);
-                    sg.load(gp + (int64_t)q0 * a.dout.stride_s, a.dout.stride_s, rows_valid, tid);
-                    sq.store(Qs, rows_valid, tid);
-                    sg.store(Gs, rows_valid, tid);
-                }
-                if (tid < BM) {
-                    const bool ok = q0 + tid < a.S;
-                    lse2s[tid] = ok ? a.lse[rowbase + q0 + tid] * kLog2e : 0.f;
-                    dls[tid] = ok ? a.delta[rowbase + q0 + tid] : 0.f;
-                    if (partial && drow) qdoc[tid] = ok ? drow[q0 + tid] : 0;
-                }
-                __syncthreads();
+    for (int n = 0; have; ++n) {
+        const int cur = n & 1;
+        const lds_ptr Qs = Qbuf(cur), Gs = Gbuf(cur);
+        MA_LDS float* lse2s = Lbuf(cur);
+        MA_LDS float* dls = Ebuf(cur);
+        MA_LDS int64_t* qdoc = Dbuf(cur);
+        if (tid < BM) {
+            lse2s[tid] = lse_next;
+            dls[tid] = dl_next;
+            if (HAS_DOC) qdoc[tid] = qd_next;
+        }
+        wait_vmem();
+        __syncthreads();
+
+        const int cq0 = q0;
+        const bool cpartial = partial;
+        have = st.next();
+        if (have) {
+            q0 = st.q0;
+            partial = st.partial;
+            issue(cur ^ 1);
+        }
 
 #pragma unroll 1
-                for (int mb = 0; mb < BM / 32; ++mb) {
-                    const int qb0 = q0 + 32 * mb;
-                    if (qb0 >= a.S) continue;
-                    if (partial && bounded && qb0 + 31 < kw_lo) continue;
-                    if (partial && a.window >= 0 && (int64_t)qb0 - kw_hi > a.window) continue;
+        for (int mb = 0; mb < BM / 32; ++mb) {
+            const int qb0 = cq0 + 32 * mb;
+            if (qb0 >= a.S) continue;
+            if (cpartial && bounded && qb0 + 31 < kw_lo) continue;
+            if (cpartial && a.window >= 0 && (int64_t)qb0 - kw_hi > a.window) continue;
 
-                    f32x16 s, dp;
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) s[v] = dp[v] = 0.f;
-#pragma unroll
-                    for (int kk = 0; kk < KK; ++kk) s = mfma32(TL::row_frag(Qs, rbase, 32 * mb, kk), kf[kk], s);
-#pragma unroll
-                    for (int kk = 0; kk < KK; ++kk) dp = mfma32(TL::row_frag(Gs, rbase, 32 * mb, kk), vf[kk], dp);
+            // S = Q K^T and dP = dO V^T for 32 q rows x the wave's 32 kv rows (lane owns one kv row)
+            f32x16 s, dp;
+            const uint32_t roff = (uint32_t)(32 * mb * TL::kPitch);
+            rowfrag_gemm2<D, kBPipe, false, false>(lds_addr(Qs) + rbase + roff, kf, s, lds_addr(Gs) + rbase + roff, vf, dp);
 
-                    bf16x8 pf[2], dsf[2];
-                    // d = q - kv for element v is drel + 8*(v/4) + v%4; all tests are branch-free
-                    const int drel = q0 + 32 * mb + 4 * hh - kv;
-                    const int dmin = bounded ? 0 : -0x40000000;
-                    const int dend = a.S - kv;                    // q < S  <=>  d < S - kv
+            bf16x8 pf[2], dsf[2];
+            // d = q - kv for element v is drel + 8*(v/4) + v%4; range test as one unsigned compare
+            const int drel = qb0 + 4 * hh - kv;
+            const int dlo = bounded ? 0 : -0x40000000;
+            const int dhi = min(wlim, a.S - 1 - kv);              // q - kv <= window, q < S
+            const unsigned span = (unsigned)(dhi - dlo);
+            const bool some = (dhi >= dlo) & kvalid;
+            const unsigned t0 = (unsigned)(drel - dlo);
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        const int qc = 8 * (v >> 2) + (v & 3);
-                        const int ql = 32 * mb + qc + 4 * hh;
-                        float p = fast_exp2(s[v] * sl2 - lse2s[ql]);
-                        if (partial) {
-                            const int d = drel + qc;
-                            bool ok = (d >= dmin) & (d <= wlim) & (d < dend) & kvalid;
-                            if (drow) ok = ok & (qdoc[ql] == dock);
-                            p = ok ? p : 0.f;
-                        }
-                        const float ds = p * (dp[v] - dls[ql]);
-                        pf[v >> 3][v & 7] = (__bf16)p;
-                        dsf[v >> 3][v & 7] = (__bf16)ds;
+            for (int g4 = 0; g4 < 4; ++g4) {
+                const int qoff = 32 * mb + 8 * g4 + 4 * hh;
+                const f32x4 l4 = *(MA_LDS f32x4*)(lse2s + qoff);
+                const f32x4 e4 = *(MA_LDS f32x4*)(dls + qoff);
+                i64x2 ida = {0, 0}, idb = {0, 0};
+                if (HAS_DOC && cpartial) {
+                    ida = *(MA_LDS i64x2*)(qdoc + qoff);
+                    idb = *(MA_LDS i64x2*)(qdoc + qoff + 2);
+                }
+                const int64_t ids[4] = {ida[0], ida[1], idb[0], idb[1]};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int v = 4 * g4 + e;
+                    float p = fast_exp2(s[v] * sl2 - l4[e]);
+                    if (cpartial) {
+                        bool ok = (t0 + (unsigned)(8 * g4 + e) <= span) & some;
+                        if (HAS_DOC) ok = ok & (ids[e] == dock);
+                        p = ok ? p : 0.f;
                     }
-#pragma unroll
-                    for (int t = 0; t < 2; ++t) {
-#pragma unroll
-                        for (int db = 0; db < DB; ++db) {
-                            dvacc[db] = mfma32(TL::tr_frag(Gs, tbase, 32 * mb + 16 * t, 32 * db), pf[t], dvacc[db]);
-                            dkacc[db] = mfma32(TL::tr_frag(Qs, tbase, 32 * mb + 16 * t, 32 * db), dsf[t], dkacc[db]);
-                        }
-                    }
+                    const float ds = p * (dp[v] - e4[e]);
+                    pf[v >> 3][v & 7] = (__bf16)p;
+                    dsf[v >> 3][v & 7] = (__bf16)ds;
                 }
             }
+            // dV^T += dO^T P and dK^T += Q^T dS  (accumulators stay in AGPRs)
+            trfrag_gemm<D, 2, kBPipe, true>(lds_addr(Gs) + tbase + roff, pf, dvacc);
+            trfrag_gemm<D, 2, kBPipe, true>(lds_addr(Qs) + tbase + roff, dsf, dkacc);
         }
     }
 
-    if (kvalid) {
-        __bf16* okp = (__bf16*)a.dk.ptr + b * a.dk.stride_b + (int64_t)kv * a.dk.stride_s + hk * a.dk.stride_h;
-        __bf16* ovp = (__bf16*)a.dv.ptr + b * a.dv.stride_b + (int64_t)kv * a.dv.stride_s + hk * a.dv.stride_h;
-#pragma unroll
-        for (int db = 0; db < DB; ++db) {
-#pragma unroll
-            for (int g4 = 0; g4 < 4; ++g4) {
-                bf16x4 pk, pv;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    pk[e] = (__bf16)(dkacc[db][4 * g4 + e] * a.scale);
-                    pv[e] = (__bf16)dvacc[db][4 * g4 + e];
-                }
-                *(bf16x4*)(okp + 32 * db + 8 * g4 + 4 * hh) = pk;
-                *(bf16x4*)(ovp + 32 * db + 8 * g4 + 4 * hh) = pv;
-            }
-        }
+    __syncthreads();  // everyone is done with the tiles: reuse the ring as store scratch
+    mfma_fence();
+    {
+        constexpr int kPitchO = D * 2 + 16;
+        const lds_ptr scratch = lds0 + w * 32 * kPitchO;
+        __bf16* okp = (__bf16*)a.dk.ptr + b * a.dk.stride_b + hk * a.dk.stride_h;
+        __bf16* ovp = (__bf16*)a.dv.ptr + b * a.dv.stride_b + hk * a.dv.stride_h;
+        store_tile_T<D>(scratch, dkacc, a.scale, okp, a.dk.stride_s, kw_lo, a.S, lane);
+        store_tile_T<D>(scratch, dvacc, 1.0f, ovp, a.dv.stride_s, kw_lo, a.S, lane);
     }
 }
 
 // ------------------------------------------------------------------------------------------------
 // dQ
 // ------------------------------------------------------------------------------------------------
-template <int D>
+struct KvStepsB {
+    const int32_t *plist, *flist;
+    int np, nf, it, half, S, q_lo, q_hi, bounded;
+    int64_t window;
+    int k0;
+    bool partial;
+
+    __device__ __forceinline__ bool next() {
+        for (;;) {
+            if (++half == kTile / kStep) {
+                half = 0;
+                ++it;
+            }
+            if (it >= np + nf) return false;
+            partial = it < np;
+            const int j = partial ? plist[it] : flist[it - np];
+            k0 = j * kTile + half * kStep;
+            if (k0 >= S) continue;
+            if (partial && bounded && k0 > q_hi) continue;
+            if (partial && window >= 0 && (int64_t)q_lo - (k0 + kStep - 1) > window) continue;
+            return true;
+        }
+    }
+};
+
+template <int D, bool HAS_DOC>
 __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dq_bf16_kernel(AttnArgs a) {
     using TL = Tile<D>;
     constexpr int KK = D / 16;
     constexpr int DB = D / 32;
     constexpr int BN = kStep;
+    constexpr int NW = kBwdThreads / 64;
     extern __shared__ __align__(16) char smem_raw[];
-    lds_ptr Ks = (lds_ptr)smem_raw;
-    lds_ptr Vs = Ks + TL::bytes(BN);
-    MA_LDS int64_t* kdoc = (MA_LDS int64_t*)(Vs + TL::bytes(BN));
+    const lds_ptr lds0 = (lds_ptr)smem_raw;
+    auto Kbuf = [&](int i) { return lds0 + i * 2 * TL::bytes(BN); };
+    auto Vbuf = [&](int i) { return lds0 + i * 2 * TL::bytes(BN) + TL::bytes(BN); };
+    auto Dbuf = [&](int i) { return (MA_LDS int64_t*)(lds0 + 4 * TL::bytes(BN)) + i * BN; };
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 31, hh = lane >> 5;
-    const int i = gridDim.y - 1 - blockIdx.y;
-    const int h = blockIdx.x % a.Hq, b = blockIdx.x / a.Hq;
+    int i, h, b;
+    map_workgroup_bwd(a, blockIdx.x, a.Hq / a.Hkv, false, i, h, b);
     const int rbase = TL::row_base(lane), tbase = TL::tr_base(lane);
     const int hk = h / (a.Hq / a.Hkv);
     const int qw_lo = i * kTile + 32 * w, qw_hi = qw_lo + 31;
@@ -233,20 +379,32 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dq_bf16_kernel(AttnArgs 
     const __bf16* gp = (const __bf16*)a.dout.ptr + b * a.dout.stride_b + h * a.dout.stride_h;
     const __bf16* kp = (const __bf16*)a.k.ptr + b * a.k.stride_b + hk * a.k.stride_h;
     const __bf16* vp = (const __bf16*)a.v.ptr + b * a.v.stride_b + hk * a.v.stride_h;
-    const int64_t* drow = a.doc ? a.doc + (size_t)b * a.S : nullptr;
-
-    const int qc = min(q, a.S - 1);  // rows past the end read the last valid row; never stored
-    bf16x8 qf[KK], gf[KK];
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-        qf[kk] = *(const bf16x8*)(qp + (int64_t)qc * a.q.stride_s + 16 * kk + 8 * hh);
-        gf[kk] = *(const bf16x8*)(gp + (int64_t)qc * a.dout.stride_s + 16 * kk + 8 * hh);
-    }
-    const int64_t docq = drow ? drow[qc] : 0;
+    const int64_t* drow = HAS_DOC ? a.doc + (size_t)b * a.S : nullptr;
+    const int qc = min(q, a.S - 1);
+    const int64_t docq = HAS_DOC ? drow[qc] : 0;
     const int wlim = a.window >= 0 ? (int)min(a.window, (int64_t)0x3fffffff) : 0x7fffffff;
     const size_t rowi = ((size_t)b * a.Hq + h) * a.S + qc;
     const float lse2 = a.lse[rowi] * kLog2e;
     const float delta = a.delta[rowi];
+
+    // Q and dO rows of the workgroup come in through LDS (coalesced) and stay in registers (AGPRs)
+    bf16x8 qf[KK], gf[KK];
+    {
+        DirectStager<D, kTile, NW> sq, sg;
+        sq.init(w, lane, a.q.stride_s);
+        sg.init(w, lane, a.dout.stride_s);
+        const int rows_valid = min(kTile, a.S - i * kTile);
+        sq.issue(qp + (int64_t)i * kTile * a.q.stride_s, Kbuf(0), w, lane, rows_valid, a.q.stride_s);
+        sg.issue(gp + (int64_t)i * kTile * a.dout.stride_s, Kbuf(1), w, lane, rows_valid, a.dout.stride_s);
+        wait_vmem();
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+            qf[kk] = TL::row_frag(Kbuf(0), rbase, 32 * w, kk);
+            gf[kk] = TL::row_frag(Kbuf(1), rbase, 32 * w, kk);
+        }
+        __syncthreads();
+    }
 
     f32x16 acc[DB];
 #pragma unroll
@@ -255,85 +413,96 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dq_bf16_kernel(AttnArgs 
         for (int v = 0; v < 16; ++v) acc[db][v] = 0.f;
 
     const size_t mrow = (size_t)b * a.T + i;
-    const int32_t* plist = a.map.kv_indices + mrow * a.T;
-    const int32_t* flist = a.map.full_kv_indices + mrow * a.T;
-    const int np = a.map.kv_num_blocks[mrow];
-    const int nf = a.map.full_kv_num_blocks[mrow];
+    KvStepsB st;
+    st.plist = a.map.kv_indices + mrow * a.T;
+    st.flist = a.map.full_kv_indices + mrow * a.T;
+    st.np = a.map.kv_num_blocks[mrow];
+    st.nf = a.map.full_kv_num_blocks[mrow];
+    st.it = 0; st.half = -1; st.S = a.S; st.q_lo = i * kTile; st.q_hi = i * kTile + kTile - 1;
+    st.bounded = bounded; st.window = a.window;
 
-    for (int it = 0; it < np + nf; ++it) {
-        const bool partial = it < np;
-        const int j = partial ? plist[it] : flist[it - np];
-        for (int half = 0; half < kTile / BN; ++half) {
-            const int k0 = j * kTile + half * BN;
-            if (k0 >= a.S) continue;
-            if (partial && bounded && k0 > i * kTile + kTile - 1) continue;
-            if (partial && a.window >= 0 && (int64_t)(i * kTile) - (k0 + BN - 1) > a.window) continue;
+    DirectStager<D, BN, NW> sk, sv;
+    sk.init(w, lane, a.k.stride_s);
+    sv.init(w, lane, a.v.stride_s);
+    int64_t kd_next = 0;
+    auto issue = [&](int buf) {
+        const int k0 = st.k0;
+        const int rows_valid = min(BN, a.S - k0);
+        sk.issue(kp + (int64_t)k0 * a.k.stride_s, Kbuf(buf), w, lane, rows_valid, a.k.stride_s);
+        sv.issue(vp + (int64_t)k0 * a.v.stride_s, Vbuf(buf), w, lane, rows_valid, a.v.stride_s);
+        if (HAS_DOC && st.partial && tid < BN) kd_next = drow[min(k0 + tid, a.S - 1)];
+    };
+    bool have = st.next();
+    int k0 = st.k0;
+    bool partial = st.partial;
+    if (have) issue(0);
 
-            __syncthreads();
-            const int rows_valid = min(BN, a.S - k0);
-            {
-                Stager<D, BN, kBwdThreads> sk, sv;
-                sk.load(kp + (int64_t)k0 * a.k.stride_s, a.k.stride_s, rows_valid, tid);
-                sv.load(vp + (int64_t)k0 * a.v.stride_s, a.v.stride_s, rows_valid, tid);
-                sk.store(Ks, rows_valid, tid);
-                sv.store(Vs, rows_valid, tid);
-            }
-            if (partial && drow && tid < BN) kdoc[tid] = (k0 + tid < a.S) ? drow[k0 + tid] : 0;
-            __syncthreads();
+    for (int n = 0; have; ++n) {
+        const int cur = n & 1;
+        const lds_ptr Ks = Kbuf(cur), Vs = Vbuf(cur);
+        MA_LDS int64_t* kdoc = Dbuf(cur);
+        if (HAS_DOC && partial && tid < BN) kdoc[tid] = kd_next;
+        wait_vmem();
+        __syncthreads();
+
+        const int ck0 = k0;
+        const bool cpartial = partial;
+        have = st.next();
+        if (have) {
+            k0 = st.k0;
+            partial = st.partial;
+            issue(cur ^ 1);
+        }
 
 #pragma unroll 1
-            for (int nb = 0; nb < BN / 32; ++nb) {
-                const int kb0 = k0 + 32 * nb;
-                if (kb0 >= a.S) continue;
-                if (partial && bounded && kb0 > qw_hi) continue;
-                if (partial && a.window >= 0 && (int64_t)qw_lo - (kb0 + 31) > a.window) continue;
+        for (int nb = 0; nb < BN / 32; ++nb) {
+            const int kb0 = ck0 + 32 * nb;
+            if (kb0 >= a.S) continue;
+            if (cpartial && bounded && kb0 > qw_hi) continue;
+            if (cpartial && a.window >= 0 && (int64_t)qw_lo - (kb0 + 31) > a.window) continue;
 
-                f32x16 s, dp;
-#pragma unroll
-                for (int v = 0; v < 16; ++v) s[v] = dp[v] = 0.f;
-#pragma unroll
-                for (int kk = 0; kk < KK; ++kk) s = mfma32(TL::row_frag(Ks, rbase, 32 * nb, kk), qf[kk], s);
-#pragma unroll
-                for (int kk = 0; kk < KK; ++kk) dp = mfma32(TL::row_frag(Vs, rbase, 32 * nb, kk), gf[kk], dp);
+            // S^T = K Q^T and dP^T = V dO^T for 32 kv rows x the wave's 32 q rows (lane owns one q row)
+            f32x16 s, dp;
+            const uint32_t roff = (uint32_t)(32 * nb * TL::kPitch);
+            rowfrag_gemm2<D, kBPipe, false, true>(lds_addr(Ks) + rbase + roff, qf, s, lds_addr(Vs) + rbase + roff, gf, dp);
 
-                bf16x8 dsf[2];
-                const int qrel = q - k0 - 32 * nb - 4 * hh;   // d = q - kv = qrel - (8*(v/4) + v%4)
-                const int dmin = bounded ? 0 : -0x40000000;
-                const int dend = q - a.S;                       // kv < S  <=>  d > q - S
+            bf16x8 dsf[2];
+            const int qrel = q - kb0 - 4 * hh;                     // d = q - kv = qrel - (8*(v/4) + v%4)
+            const int dlo = max(bounded ? 0 : -0x40000000, q - a.S + 1);
+            const unsigned span = (unsigned)(wlim - dlo);
+            const bool some = (wlim >= dlo) & qvalid;
+            const unsigned t0 = (unsigned)(qrel - dlo);
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
+            for (int g4 = 0; g4 < 4; ++g4) {
+                i64x2 ida = {0, 0}, idb = {0, 0};
+                if (HAS_DOC && cpartial) {
+                    ida = *(MA_LDS i64x2*)(kdoc + 32 * nb + 8 * g4 + 4 * hh);
+                    idb = *(MA_LDS i64x2*)(kdoc + 32 * nb + 8 * g4 + 4 * hh + 2);
+                }
+                const int64_t ids[4] = {ida[0], ida[1], idb[0], idb[1]};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int v = 4 * g4 + e;
                     float p = fast_exp2(s[v] * sl2 - lse2);
-                    if (partial) {
-                        const int kc = 8 * (v >> 2) + (v & 3);
-                        const int d = qrel - kc;
-                        bool ok = (d >= dmin) & (d <= wlim) & (d > dend) & qvalid;
-                        if (drow) ok = ok & (kdoc[32 * nb + kc + 4 * hh] == docq);
+                    if (cpartial) {
+                        bool ok = (t0 - (unsigned)(8 * g4 + e) <= span) & some;
+                        if (HAS_DOC) ok = ok & (ids[e] == docq);
                         p = ok ? p : 0.f;
                     }
                     dsf[v >> 3][v & 7] = (__bf16)(p * (dp[v] - delta));
                 }
-#pragma unroll
-                for (int t = 0; t < 2; ++t) {
-#pragma unroll
-                    for (int db = 0; db < DB; ++db)
-                        acc[db] = mfma32(TL::tr_frag(Ks, tbase, 32 * nb + 16 * t, 32 * db), dsf[t], acc[db]);
-                }
             }
+            // dQ^T += K^T dS^T  (accumulator stays in AGPRs)
+            trfrag_gemm<D, 2, kBPipe, true>(lds_addr(Ks) + tbase + roff, dsf, acc);
         }
     }
 
-    if (qvalid) {
-        __bf16* op = (__bf16*)a.dq.ptr + b * a.dq.stride_b + (int64_t)q * a.dq.stride_s + h * a.dq.stride_h;
-#pragma unroll
-        for (int db = 0; db < DB; ++db) {
-#pragma unroll
-            for (int g4 = 0; g4 < 4; ++g4) {
-                bf16x4 pk;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) pk[e] = (__bf16)(acc[db][4 * g4 + e] * a.scale);
-                *(bf16x4*)(op + 32 * db + 8 * g4 + 4 * hh) = pk;
-            }
-        }
+    __syncthreads();
+    mfma_fence();
+    {
+        constexpr int kPitchO = D * 2 + 16;
+        __bf16* ob = (__bf16*)a.dq.ptr + b * a.dq.stride_b + h * a.dq.stride_h;
+        store_tile_T<D>(lds0 + w * 32 * kPitchO, acc, a.scale, ob, a.dq.stride_s, qw_lo, a.S, lane);
     }
 }
 
@@ -345,8 +514,8 @@ static int opt_in_lds(K kernel, size_t bytes, const char* name) {
     return MA_OK;
 }
 
-template <int D>
-static int bwd_d(const AttnArgs& a, hipStream_t st) {
+template <int D, bool HAS_DOC>
+static int bwd_dd(const AttnArgs& a, hipStream_t st) {
     constexpr int RPB = 256 / (D / 8);
     const int64_t nrows = (int64_t)a.B * a.Hq * a.S;
     int rc = MA_OK;
@@ -355,22 +524,26 @@ static int bwd_d(const AttnArgs& a, hipStream_t st) {
         rc = check_launch("attn_delta_bf16_kernel");
         if (rc) return rc;
     }
-
-    const size_t lds_kv = (size_t)2 * Tile<D>::bytes(kStep) + kStep * (4 + 4 + 8);
-    rc = opt_in_lds(attn_bwd_dkv_bf16_kernel<D>, lds_kv, "attn_bwd_dkv_bf16");
-    if (rc) return rc;
     if (a.stages & MA_BWD_DKV) {
-        hipLaunchKernelGGL(attn_bwd_dkv_bf16_kernel<D>, dim3(a.B * a.Hkv, a.T, 1), dim3(kBwdThreads), lds_kv, st, a);
+        const size_t lds_kv = (size_t)4 * Tile<D>::bytes(kStep) + 2 * kStep * (4 + 4 + 8);
+        rc = opt_in_lds(attn_bwd_dkv_bf16_kernel<D, HAS_DOC>, lds_kv, "attn_bwd_dkv_bf16");
+        if (rc) return rc;
+        hipLaunchKernelGGL((attn_bwd_dkv_bf16_kernel<D, HAS_DOC>), dim3(a.B * a.Hkv * a.T, 1, 1), dim3(kBwdThreads), lds_kv,
+                           st, a);
         rc = check_launch("attn_bwd_dkv_bf16_kernel");
         if (rc) return rc;
     }
     if (!(a.stages & MA_BWD_DQ)) return MA_OK;
-
-    const size_t lds_q = (size_t)2 * Tile<D>::bytes(kStep) + kStep * 8;
-    rc = opt_in_lds(attn_bwd_dq_bf16_kernel<D>, lds_q, "attn_bwd_dq_bf16");
+    const size_t lds_q = (size_t)4 * Tile<D>::bytes(kStep) + 2 * kStep * 8;
+    rc = opt_in_lds(attn_bwd_dq_bf16_kernel<D, HAS_DOC>, lds_q, "attn_bwd_dq_bf16");
     if (rc) return rc;
-    hipLaunchKernelGGL(attn_bwd_dq_bf16_kernel<D>, dim3(a.B * a.Hq, a.T, 1), dim3(kBwdThreads), lds_q, st, a);
+    hipLaunchKernelGGL((attn_bwd_dq_bf16_kernel<D, HAS_DOC>), dim3(a.B * a.Hq * a.T, 1, 1), dim3(kBwdThreads), lds_q, st, a);
     return check_launch("attn_bwd_dq_bf16_kernel");
+}
+
+template <int D>
+static int bwd_d(const AttnArgs& a, hipStream_t st) {
+    return a.doc ? bwd_dd<D, true>(a, st) : bwd_dd<D, false>(a, st);
 }
 
 int launch_attn_bwd_bf16(const AttnArgs& a, hipStream_t st) {

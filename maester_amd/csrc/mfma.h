@@ -121,8 +121,38 @@ __device__ __forceinline__ void mfma32_av_zero(f32x16& c, bf16x8 a_agpr, bf16x8 
 __device__ __forceinline__ void mfma32_vv_zero(f32x16& c, bf16x8 a, bf16x8 b) {
     asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
 }
-// 16 wait states: enough for the result of an 8-pass MFMA to be readable by the vector ALU
+// accumulator pinned to AGPRs (for tiles no vector-ALU instruction touches inside the loop)
+__device__ __forceinline__ void mfma32_acc_a(f32x16& c, bf16x8 a, bf16x8 b) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+// 16 wait states: enough for the result of an 8-pass MFMA to be readable by the vector ALU.  The
+// tiles are read-write operands so that nothing that uses them can be scheduled above the fence
+// (volatile asm statements keep their order among themselves).
 __device__ __forceinline__ void mfma_fence() { asm volatile("s_nop 15"); }
+template <int I, int N, bool ACC_A>
+__device__ __forceinline__ void pin_tiles(f32x16* acc) {
+    if constexpr (I < N) {
+        if constexpr (ACC_A) asm volatile("" : "+a"(acc[I]));
+        else asm volatile("" : "+v"(acc[I]));
+        pin_tiles<I + 1, N, ACC_A>(acc);
+    }
+}
+// Pins N freshly computed operand fragments: everything that produces them is scheduled above this
+// point, a few wait states ahead of the MFMAs that read them (a vector-ALU result must not be
+// consumed by an MFMA in the very next cycles).
+template <int I, int N>
+__device__ __forceinline__ void pin_frags(bf16x8* f) {
+    if constexpr (I < N) {
+        if constexpr (I == 0) asm volatile("s_nop 4" : "+v"(f[0]));
+        else asm volatile("" : "+v"(f[I]));
+        pin_frags<I + 1, N>(f);
+    }
+}
+template <int N, bool ACC_A = false>
+__device__ __forceinline__ void mfma_fence_tiles(f32x16* acc) {
+    mfma_fence();
+    pin_tiles<0, N, ACC_A>(acc);
+}
 
 // ---- explicitly pipelined LDS fragment reads ---------------------------------------------------
 // The compiler serialises "LDS read -> wait -> MFMA" in these kernels, so the hot loops issue
@@ -147,14 +177,19 @@ template <int N>
 __device__ __forceinline__ void lds_wait(bf16x8& x) {
     asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(x) : "n"(N));
 }
+template <int N>
+__device__ __forceinline__ void lds_wait2(bf16x4& x, bf16x4& y) {
+    asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(x), "+v"(y) : "n"(N));
+}
 __device__ __forceinline__ uint32_t lds_addr(lds_ptr p) { return (uint32_t)(uintptr_t)p; }
 
 // acc[nb] = sum_kk L(rows 32nb + r, cols 16kk..) x reg[kk] for NB row blocks of 32 at once: a
 // software pipeline of depth P over the NB*KK row-wise fragments of an LDS tile (row_addr = lds
 // address of the tile + Tile::row_base(lane)).  The register-resident fragments reg[] live in
-// AGPRs.  SWAP puts the LDS fragment in the B slot instead (computes the transposed product).
-// acc is overwritten (no zero tile needed) and lives in VGPRs; ends with mfma_fence().
-template <int D, int NB, int P, bool SWAP = false>
+// AGPRs (REG_A) or VGPRs.  SWAP puts the LDS fragment in the B slot instead (computes the
+// transposed product).  acc is overwritten (no zero tile needed) and lives in VGPRs; ends with
+// mfma_fence().
+template <int D, int NB, int P, bool SWAP = false, bool REG_A = true>
 __device__ __forceinline__ void rowfrag_gemm(uint32_t row_addr, const bf16x8* reg, f32x16* acc) {
     using TL = Tile<D>;
     constexpr int KK = D / 16;
@@ -171,10 +206,12 @@ __device__ __forceinline__ void rowfrag_gemm(uint32_t row_addr, const bf16x8* re
         constexpr int younger = (N - 1 - i) < (P - 1) ? (N - 1 - i) : (P - 1);
         lds_wait<younger>(t[i]);
         if constexpr (kk == 0) {
-            if constexpr (SWAP) mfma32_av_zero(acc[nb], reg[kk], t[i]);
+            if constexpr (!REG_A) { if constexpr (SWAP) mfma32_vv_zero(acc[nb], reg[kk], t[i]); else mfma32_vv_zero(acc[nb], t[i], reg[kk]); }
+            else if constexpr (SWAP) mfma32_av_zero(acc[nb], reg[kk], t[i]);
             else mfma32_va_zero(acc[nb], t[i], reg[kk]);
         } else {
-            if constexpr (SWAP) mfma32_av(acc[nb], reg[kk], t[i]);
+            if constexpr (!REG_A) { if constexpr (SWAP) mfma32_vv(acc[nb], reg[kk], t[i]); else mfma32_vv(acc[nb], t[i], reg[kk]); }
+            else if constexpr (SWAP) mfma32_av(acc[nb], reg[kk], t[i]);
             else mfma32_va(acc[nb], t[i], reg[kk]);
         }
     };
@@ -184,18 +221,64 @@ __device__ __forceinline__ void rowfrag_gemm(uint32_t row_addr, const bf16x8* re
         step(idx);
         if constexpr (i + P < N) rd(std::integral_constant<int, i + P>{});
     });
+    mfma_fence_tiles<NB>(acc);
+}
+
+// Two independent products of that kind at once, from two LDS tiles, interleaved MFMA by MFMA so
+// that consecutive MFMAs never depend on each other:
+//   acc0 = sum_kk L0(rows r, cols 16kk..) x reg0[kk],  acc1 = sum_kk L1(...) x reg1[kk].
+template <int D, int P, bool SWAP = false, bool REG_A = true>
+__device__ __forceinline__ void rowfrag_gemm2(uint32_t row_addr0, const bf16x8* reg0, f32x16& acc0, uint32_t row_addr1,
+                                              const bf16x8* reg1, f32x16& acc1) {
+    constexpr int KK = D / 16;
+    constexpr int N = 2 * KK;
+    bf16x8 t[N];
+    auto rd = [&](auto idx) {
+        constexpr int i = decltype(idx)::value;
+        constexpr int kk = i / 2, which = i % 2;
+        t[i] = lds_read_b128<kk * 32>(which ? row_addr1 : row_addr0);
+    };
+    auto step = [&](auto idx) {
+        constexpr int i = decltype(idx)::value;
+        constexpr int kk = i / 2, which = i % 2;
+        constexpr int younger = (N - 1 - i) < (P - 1) ? (N - 1 - i) : (P - 1);
+        lds_wait<younger>(t[i]);
+        f32x16& acc = which ? acc1 : acc0;
+        const bf16x8 rg = which ? reg1[kk] : reg0[kk];
+        if constexpr (kk == 0) {
+            if constexpr (!REG_A) { if constexpr (SWAP) mfma32_vv_zero(acc, rg, t[i]); else mfma32_vv_zero(acc, t[i], rg); }
+            else if constexpr (SWAP) mfma32_av_zero(acc, rg, t[i]);
+            else mfma32_va_zero(acc, t[i], rg);
+        } else {
+            if constexpr (!REG_A) { if constexpr (SWAP) mfma32_vv(acc, rg, t[i]); else mfma32_vv(acc, t[i], rg); }
+            else if constexpr (SWAP) mfma32_av(acc, rg, t[i]);
+            else mfma32_va(acc, t[i], rg);
+        }
+    };
+    static_for<0, (P < N ? P : N)>(rd);
+    static_for<0, N>([&](auto idx) {
+        constexpr int i = decltype(idx)::value;
+        step(idx);
+        if constexpr (i + P < N) rd(std::integral_constant<int, i + P>{});
+    });
     mfma_fence();
+    asm volatile("" : "+v"(acc0));
+    asm volatile("" : "+v"(acc1));
 }
 
 // acc[db] += L^T(rows 16j.., cols 32db..) x reg[j] over NJ 16-row slabs of an LDS tile through
 // transposed fragments (tr_addr = lds address of the tile + Tile::tr_base(lane)).  Pipeline of
-// depth P over the NJ * DB fragments (two LDS reads each).  acc and reg live in VGPRs; ends with
-// mfma_fence().
-template <int D, int NJ, int P>
-__device__ __forceinline__ void trfrag_gemm(uint32_t tr_addr, const bf16x8* reg, f32x16* acc) {
+// depth P over the NJ * DB fragments (two LDS reads each).  reg lives in VGPRs, acc in VGPRs or
+// (ACC_A) AGPRs; ends with mfma_fence().
+template <int D, int NJ, int P, bool ACC_A = false>
+__device__ __forceinline__ void trfrag_gemm(uint32_t tr_addr, const bf16x8* reg_in, f32x16* acc) {
     using TL = Tile<D>;
     constexpr int DB = D / 32;
     constexpr int N = NJ * DB;
+    bf16x8 reg[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) reg[j] = reg_in[j];
+    pin_frags<0, NJ>(reg);
     bf16x4 lo[N], hi[N];
     auto rd = [&](auto idx) {
         constexpr int i = decltype(idx)::value;
@@ -207,9 +290,12 @@ __device__ __forceinline__ void trfrag_gemm(uint32_t tr_addr, const bf16x8* reg,
         constexpr int i = decltype(idx)::value;
         constexpr int j = i / DB, db = i % DB;
         constexpr int younger = (N - 1 - i) < (P - 1) ? (N - 1 - i) : (P - 1);
-        bf16x8 f = __builtin_shufflevector(lo[i], hi[i], 0, 1, 2, 3, 4, 5, 6, 7);
-        lds_wait<2 * younger>(f);
-        mfma32_vv(acc[db], f, reg[j]);
+        // wait on the two halves themselves: a copy made while assembling the 8-element fragment
+        // must not read them before the data has landed
+        lds_wait2<2 * younger>(lo[i], hi[i]);
+        const bf16x8 f = __builtin_shufflevector(lo[i], hi[i], 0, 1, 2, 3, 4, 5, 6, 7);
+        if constexpr (ACC_A) mfma32_acc_a(acc[db], f, reg[j]);
+        else mfma32_vv(acc[db], f, reg[j]);
     };
     static_for<0, (P < N ? P : N)>(rd);
     static_for<0, N>([&](auto idx) {
@@ -217,7 +303,7 @@ __device__ __forceinline__ void trfrag_gemm(uint32_t tr_addr, const bf16x8* reg,
         step(idx);
         if constexpr (i + P < N) rd(std::integral_constant<int, i + P>{});
     });
-    mfma_fence();  // whatever the compiler schedules next may read acc with the vector ALU
+    mfma_fence_tiles<DB, ACC_A>(acc);  // whatever comes next may read acc with the vector ALU
 }
 
 // Global -> registers -> LDS staging of a ROWS x D bf16 tile by NT threads.  load() issues all the
