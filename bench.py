@@ -80,6 +80,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c2")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 256 MiB device copy (reference point for rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is measured on ONE GPU; --gpus N with N > 1 is not run "
@@ -99,6 +101,14 @@ def main():
     wl = wl_cpu.to(dev)
     sp = wl.spec
     K, W = args.steps, args.warmup
+
+    if args.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     # ---- tile map (once per training step in the model; timed on its own) -------------------
     tmap = build_tile_map(wl.document_ids, sp.B, sp.S, True, sp.window)

@@ -250,20 +250,31 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) void prologue_bwd_kernel(
     }
 }
 
-__global__ void prologue_dw_reduce_kernel(const float* __restrict__ partials, int nblocks, int D,
-                                          float* __restrict__ dqw, float* __restrict__ dkw) {
-    const int e = blockIdx.x * blockDim.x + threadIdx.x;
-    if (e >= 2 * D) return;
+// Sums the per-block partial rows: a block owns 16 columns, 16 lanes per column stride over the rows
+// (fixed order, no atomics), then a tree over the 16 lanes in LDS.
+__global__ __launch_bounds__(256) void prologue_dw_reduce_kernel(const float* __restrict__ partials, int nblocks, int D,
+                                                                 float* __restrict__ dqw, float* __restrict__ dkw) {
+    __shared__ float red[16][17];
+    const int c = threadIdx.x & 15, rl = threadIdx.x >> 4;
+    const int e = blockIdx.x * 16 + c;
     float t = 0.f;
-    for (int r = 0; r < nblocks; ++r) t += partials[(size_t)r * 2 * D + e];
-    if (e < D) { if (dqw) dqw[e] = t; }
-    else       { if (dkw) dkw[e - D] = t; }
+    if (e < 2 * D)
+        for (int r = rl; r < nblocks; r += 16) t += partials[(size_t)r * 2 * D + e];
+    red[rl][c] = t;
+    __syncthreads();
+    if (rl == 0 && e < 2 * D) {
+        float sum = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sum += red[i][c];
+        if (e < D) { if (dqw) dqw[e] = sum; }
+        else       { if (dkw) dkw[e - D] = sum; }
+    }
 }
 
 int prologue_bwd_blocks(int B, int S) {
     const long ntok = (long)B * S;
     const long need = (ntok + kWavesPerBlock - 1) / kWavesPerBlock;
-    return (int)(need < 2048 ? need : 2048);
+    return (int)(need < 1024 ? need : 1024);
 }
 
 template <typename T, int D>
@@ -307,7 +318,7 @@ static int bwd_t(const ma_tensor4& qi, const ma_tensor4& ki, const ma_tensor4& d
                        dqi, dki, qw, kw, cs, sn, pos, n_pos, unit, q_rstd, k_rstd, partials, B, S, Hq, Hkv);
     int rc = check_launch("prologue_bwd_kernel");
     if (rc || !partials) return rc;
-    hipLaunchKernelGGL(prologue_dw_reduce_kernel, dim3((2 * D + 255) / 256), dim3(256), 0, st, partials, grid, D,
+    hipLaunchKernelGGL(prologue_dw_reduce_kernel, dim3((2 * D + 15) / 16), dim3(256), 0, st, partials, grid, D,
                        qw ? dqw : nullptr, kw ? dkw : nullptr);
     return check_launch("prologue_dw_reduce_kernel");
 }
