@@ -60,6 +60,12 @@ typedef struct ma_tile_map {
     int32_t* q_indices;          /* [B,T,T]                                          */
     int32_t* full_q_num_blocks;  /* [B,T]                                            */
     int32_t* full_q_indices;     /* [B,T,T]                                          */
+    /* Launch schedules (not part of BlockMask): the B*T q tiles (b*T + i) ordered by descending
+     * number of visited kv tiles, and the B*T kv tiles ordered by descending number of visiting q
+     * tiles.  The attention kernels start the longest-running tiles first.  Either may be NULL
+     * (natural order). */
+    int32_t* q_tile_order;       /* [B*T] */
+    int32_t* kv_tile_order;      /* [B*T] */
 } ma_tile_map;
 
 /* ---- block-sparse tile map --------------------------------------------------------------------

@@ -36,7 +36,7 @@ class MaTensor4(Structure):
 class MaTileMap(Structure):
     _fields_ = [(n, c_void_p) for n in (
         "kv_num_blocks", "kv_indices", "full_kv_num_blocks", "full_kv_indices",
-        "q_num_blocks", "q_indices", "full_q_num_blocks", "full_q_indices")]
+        "q_num_blocks", "q_indices", "full_q_num_blocks", "full_q_indices", "q_tile_order", "kv_tile_order")]
 
 
 class MaesterAttnError(RuntimeError):

@@ -22,33 +22,6 @@ namespace ma {
 constexpr int kBwdThreads = 256;
 constexpr int kStep = 64;   // rows staged per step
 constexpr int kBPipe = 4;   // LDS fragment reads kept in flight ahead of the MFMAs
-constexpr int kXcd = 8;
-
-// Workgroup id -> (tile, head, batch row) with every (batch row, kv head) pair pinned to one XCD
-// (workgroups go to the XCDs round-robin by id; each XCD has its own L2) when the pairs divide
-// evenly.  `heads` is the number of heads per kv head the grid enumerates (G for q-head grids, 1
-// for kv-head grids); `first_heavy` says whether tile 0 (true) or tile T-1 (false) is the
-// longest-running one, which is started first.
-__device__ __forceinline__ void map_workgroup_bwd(const AttnArgs& a, int id, int heads, bool first_heavy, int& tile,
-                                                  int& head, int& b) {
-    const int pairs = a.B * a.Hkv;
-    int t;
-    if (pairs % kXcd == 0) {
-        const int ppx = pairs / kXcd;
-        const int xcd = id % kXcd, n = id / kXcd;
-        t = n / (ppx * heads);
-        const int rem = n % (ppx * heads);
-        const int pair = xcd * ppx + rem / heads;
-        b = pair / a.Hkv;
-        head = (pair % a.Hkv) * heads + rem % heads;
-    } else {
-        t = id / (a.B * a.Hkv * heads);
-        const int rem = id % (a.B * a.Hkv * heads);
-        b = rem / (a.Hkv * heads);
-        head = rem % (a.Hkv * heads);
-    }
-    tile = first_heavy ? t : a.T - 1 - t;
-}
 
 // O tile epilogue shared by the kernels: a wave holds a 32-row x D fp32 tile transposed in registers
 // (lane (r, hh) owns row r and, per 32-column block, columns 8g + 4hh + e); it is scaled, cast to
@@ -159,7 +132,7 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dkv_bf16_kernel(AttnArgs
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 31, hh = lane >> 5;
     int j, hk, b;
-    map_workgroup_bwd(a, blockIdx.x, 1, true, j, hk, b);
+    if (!map_work(blockIdx.x, a.B * a.T, a.T, a.Hkv, 1, a.map.kv_tile_order, j, hk, b)) return;
     const int rbase = TL::row_base(lane), tbase = TL::tr_base(lane);
     const int G = a.Hq / a.Hkv;
     const int kw_lo = j * kTile + 32 * w, kw_hi = kw_lo + 31;
@@ -366,7 +339,7 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dq_bf16_kernel(AttnArgs 
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 31, hh = lane >> 5;
     int i, h, b;
-    map_workgroup_bwd(a, blockIdx.x, a.Hq / a.Hkv, false, i, h, b);
+    if (!map_work(blockIdx.x, a.B * a.T, a.T, a.Hkv, a.Hq / a.Hkv, a.map.q_tile_order, i, h, b)) return;
     const int rbase = TL::row_base(lane), tbase = TL::tr_base(lane);
     const int hk = h / (a.Hq / a.Hkv);
     const int qw_lo = i * kTile + 32 * w, qw_hi = qw_lo + 31;
@@ -528,7 +501,7 @@ static int bwd_dd(const AttnArgs& a, hipStream_t st) {
         const size_t lds_kv = (size_t)4 * Tile<D>::bytes(kStep) + 2 * kStep * (4 + 4 + 8);
         rc = opt_in_lds(attn_bwd_dkv_bf16_kernel<D, HAS_DOC>, lds_kv, "attn_bwd_dkv_bf16");
         if (rc) return rc;
-        hipLaunchKernelGGL((attn_bwd_dkv_bf16_kernel<D, HAS_DOC>), dim3(a.B * a.Hkv * a.T, 1, 1), dim3(kBwdThreads), lds_kv,
+        hipLaunchKernelGGL((attn_bwd_dkv_bf16_kernel<D, HAS_DOC>), dim3(work_grid(a.B * a.T, a.Hkv, 1), 1, 1), dim3(kBwdThreads), lds_kv,
                            st, a);
         rc = check_launch("attn_bwd_dkv_bf16_kernel");
         if (rc) return rc;
@@ -537,7 +510,8 @@ static int bwd_dd(const AttnArgs& a, hipStream_t st) {
     const size_t lds_q = (size_t)4 * Tile<D>::bytes(kStep) + 2 * kStep * 8;
     rc = opt_in_lds(attn_bwd_dq_bf16_kernel<D, HAS_DOC>, lds_q, "attn_bwd_dq_bf16");
     if (rc) return rc;
-    hipLaunchKernelGGL((attn_bwd_dq_bf16_kernel<D, HAS_DOC>), dim3(a.B * a.Hq * a.T, 1, 1), dim3(kBwdThreads), lds_q, st, a);
+    hipLaunchKernelGGL((attn_bwd_dq_bf16_kernel<D, HAS_DOC>), dim3(work_grid(a.B * a.T, a.Hkv, a.Hq / a.Hkv), 1, 1), dim3(kBwdThreads),
+                       lds_q, st, a);
     return check_launch("attn_bwd_dq_bf16_kernel");
 }
 

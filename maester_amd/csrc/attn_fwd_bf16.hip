@@ -50,30 +50,6 @@ struct KvSteps {
     }
 };
 
-// Workgroup id -> (q tile, q head, batch row).  Workgroups are handed to the 8 XCDs round-robin by
-// id, and each XCD has its own L2; when the (batch row, kv head) pairs divide evenly over the XCDs
-// every pair is pinned to one XCD, so the q heads and q tiles that stream the same K/V rows share
-// an L2.  Inside an XCD the late q tiles (most keys under causality) are started first.
-__device__ __forceinline__ void map_workgroup(const AttnArgs& a, int id, int& i, int& h, int& b) {
-    constexpr int kXcd = 8;
-    const int G = a.Hq / a.Hkv;
-    const int pairs = a.B * a.Hkv;
-    if (pairs % kXcd == 0) {
-        const int ppx = pairs / kXcd;  // pairs per XCD
-        const int xcd = id % kXcd, n = id / kXcd;
-        i = a.T - 1 - n / (ppx * G);
-        const int rem = n % (ppx * G);
-        const int pair = xcd * ppx + rem / G;
-        b = pair / a.Hkv;
-        h = (pair % a.Hkv) * G + rem % G;
-    } else {
-        i = a.T - 1 - id / (a.B * a.Hq);
-        const int rem = id % (a.B * a.Hq);
-        b = rem / a.Hq;
-        h = rem % a.Hq;
-    }
-}
-
 template <int D, bool HAS_DOC>
 __global__ __launch_bounds__(kFwdThreads) void attn_fwd_bf16_kernel(AttnArgs a) {
     using TL = Tile<D>;
@@ -91,7 +67,7 @@ __global__ __launch_bounds__(kFwdThreads) void attn_fwd_bf16_kernel(AttnArgs a) 
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keep it in a scalar register
     const int r = lane & 31, hh = lane >> 5;
     int i, h, b;
-    map_workgroup(a, blockIdx.x, i, h, b);
+    if (!map_work(blockIdx.x, a.B * a.T, a.T, a.Hkv, a.Hq / a.Hkv, a.map.q_tile_order, i, h, b)) return;
     const int hk = h / (a.Hq / a.Hkv);
     const int qw_lo = i * kTile + 32 * w, qw_hi = qw_lo + 31;
     const int q = qw_lo + r;
@@ -312,7 +288,8 @@ static int fwd_dd(const AttnArgs& a, hipStream_t st) {
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return fail(MA_ERR_LAUNCH, "hipFuncSetAttribute(attn_fwd_bf16, %zu): %s", lds, hipGetErrorString(e));
     }
-    hipLaunchKernelGGL((attn_fwd_bf16_kernel<D, HAS_DOC>), dim3(a.B * a.Hq * a.T, 1, 1), dim3(kFwdThreads), lds, st, a);
+    hipLaunchKernelGGL((attn_fwd_bf16_kernel<D, HAS_DOC>), dim3(work_grid(a.B * a.T, a.Hkv, a.Hq / a.Hkv), 1, 1), dim3(kFwdThreads), lds,
+                       st, a);
     return check_launch("attn_fwd_bf16_kernel");
 }
 

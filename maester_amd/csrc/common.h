@@ -61,6 +61,31 @@ int launch_attn_bwd_f32(const AttnArgs& a, hipStream_t st);
 int launch_attn_fwd_bf16(const AttnArgs& a, hipStream_t st);
 int launch_attn_bwd_bf16(const AttnArgs& a, hipStream_t st);
 
+// Workgroup id -> work item.  A unit is a tile row (q tile for the forward and dQ kernels, kv tile
+// for the dK/dV kernel) of one batch row; a combo is (unit, kv head) and owns `heads` workgroups
+// (the query heads that stream the same K/V, or 1).  Workgroups are handed to the 8 XCDs round-robin
+// by id and each XCD has its own L2, so the workgroups of one combo are given ids with the same
+// id % 8.  Units are taken in the order of `order` (descending work, from the tile map) so that the
+// longest-running workgroups start first; without it, in natural order.  Returns false for the
+// padding ids of the last group.
+constexpr int kXcds = 8;
+__host__ __device__ inline int work_grid(int n_units, int Hkv, int heads) {
+    return (n_units * Hkv + kXcds - 1) / kXcds * kXcds * heads;
+}
+__device__ __forceinline__ bool map_work(int id, int n_units, int T, int Hkv, int heads, const int32_t* order, int& tile,
+                                         int& head, int& b) {
+    const int x = id % kXcds, n = id / kXcds;
+    const int g = n % heads;
+    const int c = (n / heads) * kXcds + x;
+    if (c >= n_units * Hkv) return false;
+    const int rank = c / Hkv, hk = c % Hkv;
+    const int u = order ? order[rank] : rank;
+    b = u / T;
+    tile = u % T;
+    head = hk * heads + g;
+    return true;
+}
+
 inline int check_launch(const char* what) {
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(MA_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));

@@ -89,6 +89,31 @@ __global__ __launch_bounds__(64) void order_lists_kernel(const uint8_t* __restri
     if (lane == 0) *num = total;
 }
 
+// Launch schedule: the B*T tile rows ordered by descending work (number of tiles in the row's lists,
+// partial + full), ties by ascending index.  Block 0 orders the q tiles by their kv lists, block 1
+// the kv tiles by their q lists.  Rank by counting: N is small (B*T), the keys sit in LDS.
+constexpr int kSchedMax = 8192;
+__global__ __launch_bounds__(1024) void schedule_kernel(int N, ma_tile_map out) {
+    __shared__ int key[kSchedMax];
+    const bool qside = blockIdx.x == 0;
+    int32_t* dst = qside ? out.q_tile_order : out.kv_tile_order;
+    if (!dst) return;
+    if (N > kSchedMax) {  // too many rows to rank here: natural order
+        for (int e = threadIdx.x; e < N; e += blockDim.x) dst[e] = e;
+        return;
+    }
+    const int32_t* na = qside ? out.kv_num_blocks : out.q_num_blocks;
+    const int32_t* nb = qside ? out.full_kv_num_blocks : out.full_q_num_blocks;
+    for (int e = threadIdx.x; e < N; e += blockDim.x) key[e] = na[e] + nb[e];
+    __syncthreads();
+    for (int e = threadIdx.x; e < N; e += blockDim.x) {
+        const int k = key[e];
+        int rank = 0;
+        for (int f = 0; f < N; ++f) rank += (key[f] > k) | ((key[f] == k) & (f < e));
+        dst[rank] = e;
+    }
+}
+
 int launch_tile_map(const int64_t* doc, int B, int S, int causal, int64_t window, const ma_tile_map& out,
                     void* ws, hipStream_t st) {
     const int T = (S + kTile - 1) / kTile;
@@ -97,7 +122,10 @@ int launch_tile_map(const int64_t* doc, int B, int S, int causal, int64_t window
     int rc = check_launch("classify_tiles_kernel");
     if (rc) return rc;
     hipLaunchKernelGGL(order_lists_kernel, dim3(T, B, 4), dim3(64), 0, st, cls, T, out);
-    return check_launch("order_lists_kernel");
+    rc = check_launch("order_lists_kernel");
+    if (rc || (!out.q_tile_order && !out.kv_tile_order)) return rc;
+    hipLaunchKernelGGL(schedule_kernel, dim3(2), dim3(1024), 0, st, B * T, out);
+    return check_launch("schedule_kernel");
 }
 
 }  // namespace ma

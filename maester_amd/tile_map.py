@@ -33,6 +33,9 @@ class TileMap:
     causal: bool
     window: int | None
     BLOCK_SIZE: tuple = (TILE, TILE)
+    # launch schedules (not part of BlockMask): tile rows b*T+i by descending work, int32 [B*T]
+    q_tile_order: torch.Tensor | None = None
+    kv_tile_order: torch.Tensor | None = None
 
     NAMES = ("kv_num_blocks", "kv_indices", "full_kv_num_blocks", "full_kv_indices",
              "q_num_blocks", "q_indices", "full_q_num_blocks", "full_q_indices")
@@ -41,7 +44,9 @@ class TileMap:
         return {n: getattr(self, n) for n in self.NAMES}
 
     def c_struct(self) -> _lib.MaTileMap:
-        return _lib.MaTileMap(*[c_void_p(getattr(self, n).data_ptr()) for n in self.NAMES])
+        ptrs = [c_void_p(getattr(self, n).data_ptr()) for n in self.NAMES]
+        ptrs += [None if t is None else c_void_p(t.data_ptr()) for t in (self.q_tile_order, self.kv_tile_order)]
+        return _lib.MaTileMap(*ptrs)
 
     @property
     def seq_lengths(self):
@@ -72,8 +77,10 @@ def build_tile_map(document_ids: torch.Tensor | None, batch_size: int, seq_len: 
     T = (seq_len + TILE - 1) // TILE
     nums = torch.empty(4, batch_size, 1, T, dtype=torch.int32, device=device)
     idxs = torch.empty(4, batch_size, 1, T, T, dtype=torch.int32, device=device)
+    order = torch.empty(2, batch_size * T, dtype=torch.int32, device=device)
     tm = TileMap(nums[0], idxs[0], nums[1], idxs[1], nums[2], idxs[2], nums[3], idxs[3],
-                 seq_len=seq_len, causal=bool(causal), window=sliding_window)
+                 seq_len=seq_len, causal=bool(causal), window=sliding_window, q_tile_order=order[0],
+                 kv_tile_order=order[1])
     ws_bytes = L.ma_tile_map_workspace_bytes(batch_size, seq_len)
     ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=device)
     cs = tm.c_struct()
