@@ -72,3 +72,23 @@ def test_padding_tail_and_large_T(gpu):
     ids = torch.zeros((1, S), dtype=torch.long)
     ids[:, 5000:12000] = 1; ids[:, 12000:] = 2
     _assert_equal(build_tile_map(ids.to(gpu), 1, S, True, 4096), otm.tile_lists_c(ids, 1, S, True, 4096), "T=151")
+
+
+def _expected_order(num_a, num_b):
+    """The launch-schedule rule restated: rows by descending work (tiles in the row's lists, partial
+    + full), ties by ascending index."""
+    work = (num_a + num_b).reshape(-1)
+    return np.array(sorted(range(work.size), key=lambda e: (-work[e], e)), dtype=np.int32)
+
+
+@pytest.mark.parametrize("name,S", [("c2", 8192), ("c3", 8192), ("c1", 2048), ("c2", 1000)])
+def test_launch_schedule_orders(gpu, name, S):
+    wl = workloads.make(name, S=S)
+    sp = wl.spec
+    tm = build_tile_map(wl.document_ids.to(gpu), sp.B, sp.S, True, sp.window)
+    T = (sp.S + 127) // 128
+    d = {k: v.cpu().numpy() for k, v in tm.as_dict().items()}
+    q_order, kv_order = tm.q_tile_order.cpu().numpy(), tm.kv_tile_order.cpu().numpy()
+    assert sorted(q_order.tolist()) == list(range(sp.B * T)) and sorted(kv_order.tolist()) == list(range(sp.B * T))
+    assert np.array_equal(q_order, _expected_order(d["kv_num_blocks"], d["full_kv_num_blocks"]))
+    assert np.array_equal(kv_order, _expected_order(d["q_num_blocks"], d["full_q_num_blocks"]))
