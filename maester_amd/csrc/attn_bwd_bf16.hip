@@ -84,25 +84,20 @@ __global__ __launch_bounds__(256) void attn_delta_bf16_kernel(AttnArgs a) {
 // Walks, for each of the G query heads of the kv head, the (partial, then full) q tile lists of one
 // kv tile in steps of kStep q rows, skipping steps no row of the workgroup can see.
 struct QSteps {
-    const int32_t *plist, *flist;
-    int np, nf, G, g, it, half, S, k_lo, k_hi, bounded;
+    ListWalk walk;
+    int half, S, k_lo, k_hi, bounded, zero, tile;
     int64_t window;
     int q0;
     bool partial;
 
+    __device__ __forceinline__ int g() const { return walk.rep; }
     __device__ __forceinline__ bool next() {
         for (;;) {
             if (++half == kTile / kStep) {
                 half = 0;
-                if (++it >= np + nf) {
-                    it = 0;
-                    ++g;
-                }
+                if (!walk.advance(tile, partial, zero)) return false;
             }
-            if (g >= G || np + nf == 0) return false;
-            partial = it < np;
-            const int i = partial ? plist[it] : flist[it - np];
-            q0 = i * kTile + half * kStep;
+            q0 = tile * kTile + half * kStep;
             if (q0 >= S) continue;
             if (partial && bounded && q0 + kStep - 1 < k_lo) continue;
             if (partial && window >= 0 && (int64_t)q0 - k_hi > window) continue;
@@ -175,11 +170,10 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dkv_bf16_kernel(AttnArgs
 
     const size_t mrow = (size_t)b * a.T + j;
     QSteps st;
-    st.plist = a.map.q_indices + mrow * a.T;
-    st.flist = a.map.full_q_indices + mrow * a.T;
-    st.np = a.map.q_num_blocks[mrow];
-    st.nf = a.map.full_q_num_blocks[mrow];
-    st.G = G; st.g = 0; st.it = 0; st.half = -1; st.S = a.S;
+    st.zero = opaque_lane_zero();
+    st.walk.init(a.map.q_indices + mrow * a.T, a.map.q_num_blocks[mrow], a.map.full_q_indices + mrow * a.T,
+                 a.map.full_q_num_blocks[mrow], G, st.zero);
+    st.half = kTile / kStep - 1; st.tile = 0; st.partial = false; st.S = a.S;
     st.k_lo = j * kTile; st.k_hi = j * kTile + kTile - 1; st.bounded = bounded; st.window = a.window;
 
     DirectStager<D, BM, NW> sq, sg;
@@ -188,7 +182,7 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dkv_bf16_kernel(AttnArgs
     float lse_next = 0.f, dl_next = 0.f;
     int64_t qd_next = 0;
     auto issue = [&](int buf) {
-        const int h = hk * G + st.g;
+        const int h = hk * G + st.g();
         const int q0 = st.q0;
         const int rows_valid = min(BM, a.S - q0);
         const __bf16* qp = (const __bf16*)a.q.ptr + b * a.q.stride_b + h * a.q.stride_h + (int64_t)q0 * a.q.stride_s;
@@ -198,7 +192,7 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dkv_bf16_kernel(AttnArgs
         if (tid < BM) {
             const int qq = min(q0 + tid, a.S - 1);
             const size_t row = ((size_t)b * a.Hq + h) * a.S + qq;
-            lse_next = a.lse[row] * kLog2e;
+            lse_next = a.lse[row];  // converted to log2 units when it is written to LDS
             dl_next = a.delta[row];
             if (HAS_DOC) qd_next = drow[qq];
         }
@@ -215,7 +209,7 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dkv_bf16_kernel(AttnArgs
         MA_LDS float* dls = Ebuf(cur);
         MA_LDS int64_t* qdoc = Dbuf(cur);
         if (tid < BM) {
-            lse2s[tid] = lse_next;
+            lse2s[tid] = lse_next * kLog2e;
             dls[tid] = dl_next;
             if (HAS_DOC) qdoc[tid] = qd_next;
         }
@@ -298,8 +292,8 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dkv_bf16_kernel(AttnArgs
 // dQ
 // ------------------------------------------------------------------------------------------------
 struct KvStepsB {
-    const int32_t *plist, *flist;
-    int np, nf, it, half, S, q_lo, q_hi, bounded;
+    ListWalk walk;
+    int half, S, q_lo, q_hi, bounded, zero, tile;
     int64_t window;
     int k0;
     bool partial;
@@ -308,12 +302,9 @@ struct KvStepsB {
         for (;;) {
             if (++half == kTile / kStep) {
                 half = 0;
-                ++it;
+                if (!walk.advance(tile, partial, zero)) return false;
             }
-            if (it >= np + nf) return false;
-            partial = it < np;
-            const int j = partial ? plist[it] : flist[it - np];
-            k0 = j * kTile + half * kStep;
+            k0 = tile * kTile + half * kStep;
             if (k0 >= S) continue;
             if (partial && bounded && k0 > q_hi) continue;
             if (partial && window >= 0 && (int64_t)q_lo - (k0 + kStep - 1) > window) continue;
@@ -387,11 +378,11 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dq_bf16_kernel(AttnArgs 
 
     const size_t mrow = (size_t)b * a.T + i;
     KvStepsB st;
-    st.plist = a.map.kv_indices + mrow * a.T;
-    st.flist = a.map.full_kv_indices + mrow * a.T;
-    st.np = a.map.kv_num_blocks[mrow];
-    st.nf = a.map.full_kv_num_blocks[mrow];
-    st.it = 0; st.half = -1; st.S = a.S; st.q_lo = i * kTile; st.q_hi = i * kTile + kTile - 1;
+    st.zero = opaque_lane_zero();
+    st.walk.init(a.map.kv_indices + mrow * a.T, a.map.kv_num_blocks[mrow], a.map.full_kv_indices + mrow * a.T,
+                 a.map.full_kv_num_blocks[mrow], 1, st.zero);
+    st.half = kTile / kStep - 1; st.tile = 0; st.partial = false; st.S = a.S;
+    st.q_lo = i * kTile; st.q_hi = i * kTile + kTile - 1;
     st.bounded = bounded; st.window = a.window;
 
     DirectStager<D, BN, NW> sk, sv;

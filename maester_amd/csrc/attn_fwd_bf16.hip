@@ -26,8 +26,8 @@ constexpr int kPipe = 4;  // LDS fragment reads kept in flight ahead of the MFMA
 // Walks the (partial, then full) kv tile lists of one q tile in steps of BN rows, skipping the
 // steps no row of the workgroup can see.  All state is workgroup-uniform.
 struct KvSteps {
-    const int32_t *plist, *flist;
-    int np, nf, it, half, S, q_lo, q_hi, bounded;
+    ListWalk walk;
+    int half, S, q_lo, q_hi, bounded, zero, tile;
     int64_t window;
     int k0;
     bool partial;
@@ -36,12 +36,9 @@ struct KvSteps {
         for (;;) {
             if (++half == kTile / kFwdBN) {
                 half = 0;
-                ++it;
+                if (!walk.advance(tile, partial, zero)) return false;
             }
-            if (it >= np + nf) return false;
-            partial = it < np;
-            const int j = partial ? plist[it] : flist[it - np];
-            k0 = j * kTile + half * kFwdBN;
+            k0 = tile * kTile + half * kFwdBN;
             if (k0 >= S) continue;
             if (partial && bounded && k0 > q_hi) continue;
             if (partial && window >= 0 && (int64_t)q_lo - (k0 + kFwdBN - 1) > window) continue;
@@ -95,11 +92,11 @@ __global__ __launch_bounds__(kFwdThreads) void attn_fwd_bf16_kernel(AttnArgs a) 
 
     const size_t mrow = (size_t)b * a.T + i;
     KvSteps st;
-    st.plist = a.map.kv_indices + mrow * a.T;
-    st.flist = a.map.full_kv_indices + mrow * a.T;
-    st.np = a.map.kv_num_blocks[mrow];
-    st.nf = a.map.full_kv_num_blocks[mrow];
-    st.it = 0; st.half = -1; st.S = a.S; st.q_lo = i * kTile; st.q_hi = i * kTile + kTile - 1;
+    st.zero = opaque_lane_zero();
+    st.walk.init(a.map.kv_indices + mrow * a.T, a.map.kv_num_blocks[mrow], a.map.full_kv_indices + mrow * a.T,
+                 a.map.full_kv_num_blocks[mrow], 1, st.zero);
+    st.half = kTile / kFwdBN - 1; st.tile = 0; st.partial = false; st.S = a.S;
+    st.q_lo = i * kTile; st.q_hi = i * kTile + kTile - 1;
     st.bounded = bounded; st.window = a.window;
 
     DirectStager<D, BN, kFwdThreads / 64> sk, sv;

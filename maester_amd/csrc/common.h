@@ -86,6 +86,41 @@ __device__ __forceinline__ bool map_work(int id, int n_units, int T, int Hkv, in
     return true;
 }
 
+// Walks `reps` times over the concatenation of two tile lists (partial tiles, then full tiles) of a
+// tile-map row.  The index of the following entry is always in flight: it is loaded when the current
+// one is handed out and only read (readfirstlane) a whole step later, so the walk never waits on
+// memory.  `zero` must be a per-lane zero the compiler cannot see through (it keeps the load a plain
+// per-lane load whose result stays in a vector register until it is needed).
+struct ListWalk {
+    const int32_t *pl, *fl;
+    int np, n, reps, rep, it;
+    int nxt;
+
+    __device__ __forceinline__ int fetch(int i, int zero) const { return i < np ? pl[i + zero] : fl[i - np + zero]; }
+    __device__ __forceinline__ void init(const int32_t* partial_list, int n_partial, const int32_t* full_list, int n_full,
+                                         int repeats, int zero) {
+        pl = partial_list; fl = full_list; np = n_partial; n = n_partial + n_full; reps = repeats;
+        rep = 0; it = -1;
+        nxt = n ? fetch(0, zero) : 0;
+    }
+    __device__ __forceinline__ bool advance(int& tile, bool& partial, int zero) {
+        if (n == 0) return false;
+        if (++it == n) {
+            it = 0;
+            if (++rep == reps) return false;
+        }
+        tile = __builtin_amdgcn_readfirstlane(nxt);
+        partial = it < np;
+        nxt = fetch(it + 1 == n ? 0 : it + 1, zero);
+        return true;
+    }
+};
+__device__ __forceinline__ int opaque_lane_zero() {
+    int z;
+    asm volatile("v_mov_b32 %0, 0" : "=v"(z));
+    return z;
+}
+
 inline int check_launch(const char* what) {
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(MA_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));

@@ -189,8 +189,16 @@ __device__ __forceinline__ uint32_t lds_addr(lds_ptr p) { return (uint32_t)(uint
 // AGPRs (REG_A) or VGPRs.  SWAP puts the LDS fragment in the B slot instead (computes the
 // transposed product).  acc is overwritten (no zero tile needed) and lives in VGPRs; ends with
 // mfma_fence().
-template <int D, int NB, int P, bool SWAP = false, bool REG_A = true>
-__device__ __forceinline__ void rowfrag_gemm(uint32_t row_addr, const bf16x8* reg, f32x16* acc) {
+struct NoHook {
+    template <typename I>
+    __device__ __forceinline__ void operator()(I) const {}
+};
+
+// hook(integral_constant<int, i>) runs right after MFMA i has been issued: the kernels use it to
+// spread the global -> LDS loads of the next step over the chain instead of issuing them in one
+// burst (a burst fills the memory pipeline and stalls the wave with the matrix cores idle).
+template <int D, int NB, int P, bool SWAP = false, bool REG_A = true, typename Hook = NoHook>
+__device__ __forceinline__ void rowfrag_gemm(uint32_t row_addr, const bf16x8* reg, f32x16* acc, Hook&& hook = Hook{}) {
     using TL = Tile<D>;
     constexpr int KK = D / 16;
     constexpr int N = NB * KK;
@@ -220,6 +228,7 @@ __device__ __forceinline__ void rowfrag_gemm(uint32_t row_addr, const bf16x8* re
         constexpr int i = decltype(idx)::value;
         step(idx);
         if constexpr (i + P < N) rd(std::integral_constant<int, i + P>{});
+        hook(idx);
     });
     mfma_fence_tiles<NB>(acc);
 }
@@ -227,9 +236,9 @@ __device__ __forceinline__ void rowfrag_gemm(uint32_t row_addr, const bf16x8* re
 // Two independent products of that kind at once, from two LDS tiles, interleaved MFMA by MFMA so
 // that consecutive MFMAs never depend on each other:
 //   acc0 = sum_kk L0(rows r, cols 16kk..) x reg0[kk],  acc1 = sum_kk L1(...) x reg1[kk].
-template <int D, int P, bool SWAP = false, bool REG_A = true>
+template <int D, int P, bool SWAP = false, bool REG_A = true, typename Hook = NoHook>
 __device__ __forceinline__ void rowfrag_gemm2(uint32_t row_addr0, const bf16x8* reg0, f32x16& acc0, uint32_t row_addr1,
-                                              const bf16x8* reg1, f32x16& acc1) {
+                                              const bf16x8* reg1, f32x16& acc1, Hook&& hook = Hook{}) {
     constexpr int KK = D / 16;
     constexpr int N = 2 * KK;
     bf16x8 t[N];
@@ -260,6 +269,7 @@ __device__ __forceinline__ void rowfrag_gemm2(uint32_t row_addr0, const bf16x8* 
         constexpr int i = decltype(idx)::value;
         step(idx);
         if constexpr (i + P < N) rd(std::integral_constant<int, i + P>{});
+        hook(idx);
     });
     mfma_fence();
     asm volatile("" : "+v"(acc0));
@@ -270,8 +280,8 @@ __device__ __forceinline__ void rowfrag_gemm2(uint32_t row_addr0, const bf16x8* 
 // transposed fragments (tr_addr = lds address of the tile + Tile::tr_base(lane)).  Pipeline of
 // depth P over the NJ * DB fragments (two LDS reads each).  reg lives in VGPRs, acc in VGPRs or
 // (ACC_A) AGPRs; ends with mfma_fence().
-template <int D, int NJ, int P, bool ACC_A = false>
-__device__ __forceinline__ void trfrag_gemm(uint32_t tr_addr, const bf16x8* reg_in, f32x16* acc) {
+template <int D, int NJ, int P, bool ACC_A = false, typename Hook = NoHook>
+__device__ __forceinline__ void trfrag_gemm(uint32_t tr_addr, const bf16x8* reg_in, f32x16* acc, Hook&& hook = Hook{}) {
     using TL = Tile<D>;
     constexpr int DB = D / 32;
     constexpr int N = NJ * DB;
@@ -302,6 +312,7 @@ __device__ __forceinline__ void trfrag_gemm(uint32_t tr_addr, const bf16x8* reg_
         constexpr int i = decltype(idx)::value;
         step(idx);
         if constexpr (i + P < N) rd(std::integral_constant<int, i + P>{});
+        hook(idx);
     });
     mfma_fence_tiles<DB, ACC_A>(acc);  // whatever comes next may read acc with the vector ALU
 }
@@ -345,6 +356,15 @@ struct Stager {
 // (row, chunk) lands in a slot is decided on the global side, so the permuted/padded layout costs
 // nothing.  Rows at or beyond rows_valid re-read the last valid row (callers mask them).
 #define MA_GLB __attribute__((address_space(1)))
+// One run: 64 lanes x 16 bytes from (wave-uniform base + per-lane byte offset) to LDS at the
+// wave-uniform address lds .. lds + 1023.  An asm statement so that it keeps its place among the
+// MFMAs and LDS reads of a chain (which are asm statements too).
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"  // m0 is clobbered on purpose: it carries the LDS address
+__device__ __forceinline__ void global_to_lds_run(const void* base, uint32_t voff, uint32_t lds) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds), "v"(voff), "s"(base) : "m0");
+}
+#pragma clang diagnostic pop
 template <int D, int ROWS, int NWAVES>
 struct DirectStager {
     using TL = Tile<D>;
@@ -362,13 +382,21 @@ struct DirectStager {
         if (chunk == TL::kChunks) chunk = 0;
         row = TL::prow(rho);  // prow is its own inverse
     }
+    // run p of wave w; when the runs do not divide evenly the surplus slots of the last round repeat
+    // the last run (same data to the same place), so that every wave issues the same instructions
+    __device__ __forceinline__ static int run_of(int w, int p) { return min(w + p * NWAVES, NL - 1); }
     __device__ __forceinline__ void init(int w, int lane, int64_t stride) {
 #pragma unroll
         for (int p = 0; p < PER; ++p) {
             int row, chunk;
-            slot(w + p * NWAVES, lane, row, chunk);
+            slot(run_of(w, p), lane, row, chunk);
             off[p] = (uint32_t)((row * stride + chunk * 8) * 2);
         }
+    }
+    // run P of this wave for a whole tile (all ROWS rows valid)
+    template <int P>
+    __device__ __forceinline__ void issue_one(const __bf16* g, uint32_t tile_addr, int w) const {
+        if constexpr (P < PER) global_to_lds_run(g, off[P], tile_addr + run_of(w, P) * 1024);
     }
     __device__ __forceinline__ void issue(const __bf16* g, lds_ptr tile, int w, int lane, int rows_valid,
                                           int64_t stride) const {
