@@ -147,8 +147,8 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dkv_bf16_kernel(AttnArgs
     bf16x8 kf[KK], vf[KK];
     {
         DirectStager<D, kTile, NW> sk, sv;
-        sk.init(w, lane, a.k.stride_s);
-        sv.init(w, lane, a.v.stride_s);
+        sk.init(w, lane);
+        sv.init(w, lane);
         const int rows_valid = min(kTile, a.S - j * kTile);
         sk.issue(kp + (int64_t)j * kTile * a.k.stride_s, Qbuf(0), w, lane, rows_valid, a.k.stride_s);
         sv.issue(vp + (int64_t)j * kTile * a.v.stride_s, Qbuf(1), w, lane, rows_valid, a.v.stride_s);
@@ -172,35 +172,44 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dkv_bf16_kernel(AttnArgs
     QSteps st;
     st.zero = opaque_lane_zero();
     st.walk.init(a.map.q_indices + mrow * a.T, a.map.q_num_blocks[mrow], a.map.full_q_indices + mrow * a.T,
-                 a.map.full_q_num_blocks[mrow], G, st.zero);
+                 a.map.full_q_num_blocks[mrow], G, true, st.zero);
     st.half = kTile / kStep - 1; st.tile = 0; st.partial = false; st.S = a.S;
     st.k_lo = j * kTile; st.k_hi = j * kTile + kTile - 1; st.bounded = bounded; st.window = a.window;
 
     DirectStager<D, BM, NW> sq, sg;
-    sq.init(w, lane, a.q.stride_s);
-    sg.init(w, lane, a.dout.stride_s);
+    sq.init(w, lane);
+    sg.init(w, lane);
     float lse_next = 0.f, dl_next = 0.f;
     int64_t qd_next = 0;
-    auto issue = [&](int buf) {
+    // global sources of the step the iterator stands on
+    const __bf16 *qsrc = nullptr, *gsrc = nullptr;
+    auto locate = [&]() {
         const int h = hk * G + st.g();
-        const int q0 = st.q0;
-        const int rows_valid = min(BM, a.S - q0);
-        const __bf16* qp = (const __bf16*)a.q.ptr + b * a.q.stride_b + h * a.q.stride_h + (int64_t)q0 * a.q.stride_s;
-        const __bf16* gp = (const __bf16*)a.dout.ptr + b * a.dout.stride_b + h * a.dout.stride_h + (int64_t)q0 * a.dout.stride_s;
-        sq.issue(qp, Qbuf(buf), w, lane, rows_valid, a.q.stride_s);
-        sg.issue(gp, Gbuf(buf), w, lane, rows_valid, a.dout.stride_s);
+        qsrc = (const __bf16*)a.q.ptr + b * a.q.stride_b + h * a.q.stride_h + (int64_t)st.q0 * a.q.stride_s;
+        gsrc = (const __bf16*)a.dout.ptr + b * a.dout.stride_b + h * a.dout.stride_h + (int64_t)st.q0 * a.dout.stride_s;
+    };
+    auto issue_rows = [&]() {  // per-row lse / delta / document id of that step
         if (tid < BM) {
-            const int qq = min(q0 + tid, a.S - 1);
+            const int h = hk * G + st.g();
+            const int qq = min(st.q0 + tid, a.S - 1);
             const size_t row = ((size_t)b * a.Hq + h) * a.S + qq;
             lse_next = a.lse[row];  // converted to log2 units when it is written to LDS
             dl_next = a.delta[row];
             if (HAS_DOC) qd_next = drow[qq];
         }
     };
+    auto issue_q = [&](int buf) { sq.issue(qsrc, Qbuf(buf), w, lane, min(BM, a.S - st.q0), a.q.stride_s); };
+    auto issue_g = [&](int buf) { sg.issue(gsrc, Gbuf(buf), w, lane, min(BM, a.S - st.q0), a.dout.stride_s); };
+    const int my_runs = decltype(sq)::runs_of(w);
     bool have = st.next();
     int q0 = st.q0;
     bool partial = st.partial;
-    if (have) issue(0);
+    if (have) {
+        locate();
+        issue_q(0);
+        issue_g(0);
+        issue_rows();
+    }
 
     for (int n = 0; have; ++n) {
         const int cur = n & 1;
@@ -219,23 +228,51 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dkv_bf16_kernel(AttnArgs
         const int cq0 = q0;
         const bool cpartial = partial;
         have = st.next();
+        // The tile loads of the next step are spread over this step's first MFMA chains, one run
+        // every few MFMAs (Q tile in the first 32-row block, dO tile in the second): issued in one
+        // burst they fill the memory pipeline and stall the wave with the matrix cores idle.  A
+        // ragged last tile, or a block that is skipped, issues its tile at once.
+        bool skip[BM / 32];
+#pragma unroll
+        for (int mb = 0; mb < BM / 32; ++mb) {
+            const int qb0 = cq0 + 32 * mb;
+            skip[mb] = qb0 >= a.S;
+            if (cpartial && bounded && qb0 + 31 < kw_lo) skip[mb] = true;
+            if (cpartial && a.window >= 0 && (int64_t)qb0 - kw_hi > a.window) skip[mb] = true;
+        }
+        int pace = 0;
         if (have) {
             q0 = st.q0;
             partial = st.partial;
-            issue(cur ^ 1);
+            locate();
+            issue_rows();
+            const bool spread = (q0 + BM <= a.S) & !skip[0] & !skip[1];
+            pace = __builtin_amdgcn_readfirstlane(spread ? my_runs : 0);
+            if (!pace) {
+                issue_q(cur ^ 1);
+                issue_g(cur ^ 1);
+            }
         }
+        const uint32_t qdst = lds_addr(Qbuf(cur ^ 1)), gdst = lds_addr(Gbuf(cur ^ 1));
+        const uint32_t qsb = (uint32_t)(a.q.stride_s * 2), gsb = (uint32_t)(a.dout.stride_s * 2);
 
 #pragma unroll 1
         for (int mb = 0; mb < BM / 32; ++mb) {
             const int qb0 = cq0 + 32 * mb;
-            if (qb0 >= a.S) continue;
-            if (cpartial && bounded && qb0 + 31 < kw_lo) continue;
-            if (cpartial && a.window >= 0 && (int64_t)qb0 - kw_hi > a.window) continue;
+            if (mb ? skip[1] : skip[0]) continue;
+            const __bf16* psrc = mb ? gsrc : qsrc;
+            const uint32_t pdst = mb ? gdst : qdst, psb = mb ? gsb : qsb;
+            constexpr int kEvery = (2 * KK) / decltype(sq)::PER;
+            static_assert(kEvery >= 1, "pacing");
+            auto pace_hook = [&](auto idx) {
+                constexpr int i = decltype(idx)::value;
+                if constexpr (i % kEvery == kEvery - 1) sq.template issue_one<i / kEvery>(psrc, pdst, w, pace, psb);
+            };
 
             // S = Q K^T and dP = dO V^T for 32 q rows x the wave's 32 kv rows (lane owns one kv row)
             f32x16 s, dp;
             const uint32_t roff = (uint32_t)(32 * mb * TL::kPitch);
-            rowfrag_gemm2<D, kBPipe, false, false>(lds_addr(Qs) + rbase + roff, kf, s, lds_addr(Gs) + rbase + roff, vf, dp);
+            rowfrag_gemm2<D, kBPipe, false, false>(lds_addr(Qs) + rbase + roff, kf, s, lds_addr(Gs) + rbase + roff, vf, dp, pace_hook);
 
             bf16x8 pf[2], dsf[2];
             // d = q - kv for element v is drel + 8*(v/4) + v%4; range test as one unsigned compare
@@ -355,8 +392,8 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dq_bf16_kernel(AttnArgs 
     bf16x8 qf[KK], gf[KK];
     {
         DirectStager<D, kTile, NW> sq, sg;
-        sq.init(w, lane, a.q.stride_s);
-        sg.init(w, lane, a.dout.stride_s);
+        sq.init(w, lane);
+        sg.init(w, lane);
         const int rows_valid = min(kTile, a.S - i * kTile);
         sq.issue(qp + (int64_t)i * kTile * a.q.stride_s, Kbuf(0), w, lane, rows_valid, a.q.stride_s);
         sg.issue(gp + (int64_t)i * kTile * a.dout.stride_s, Kbuf(1), w, lane, rows_valid, a.dout.stride_s);
@@ -380,26 +417,34 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dq_bf16_kernel(AttnArgs 
     KvStepsB st;
     st.zero = opaque_lane_zero();
     st.walk.init(a.map.kv_indices + mrow * a.T, a.map.kv_num_blocks[mrow], a.map.full_kv_indices + mrow * a.T,
-                 a.map.full_kv_num_blocks[mrow], 1, st.zero);
+                 a.map.full_kv_num_blocks[mrow], 1, false, st.zero);
     st.half = kTile / kStep - 1; st.tile = 0; st.partial = false; st.S = a.S;
     st.q_lo = i * kTile; st.q_hi = i * kTile + kTile - 1;
     st.bounded = bounded; st.window = a.window;
 
     DirectStager<D, BN, NW> sk, sv;
-    sk.init(w, lane, a.k.stride_s);
-    sv.init(w, lane, a.v.stride_s);
+    sk.init(w, lane);
+    sv.init(w, lane);
     int64_t kd_next = 0;
-    auto issue = [&](int buf) {
-        const int k0 = st.k0;
-        const int rows_valid = min(BN, a.S - k0);
-        sk.issue(kp + (int64_t)k0 * a.k.stride_s, Kbuf(buf), w, lane, rows_valid, a.k.stride_s);
-        sv.issue(vp + (int64_t)k0 * a.v.stride_s, Vbuf(buf), w, lane, rows_valid, a.v.stride_s);
-        if (HAS_DOC && st.partial && tid < BN) kd_next = drow[min(k0 + tid, a.S - 1)];
+    // the step the iterator stands on
+    auto issue_k = [&](int buf) {
+        sk.issue(kp + (int64_t)st.k0 * a.k.stride_s, Kbuf(buf), w, lane, min(BN, a.S - st.k0), a.k.stride_s);
     };
+    auto issue_v = [&](int buf) {
+        sv.issue(vp + (int64_t)st.k0 * a.v.stride_s, Vbuf(buf), w, lane, min(BN, a.S - st.k0), a.v.stride_s);
+    };
+    auto issue_ids = [&]() {
+        if (HAS_DOC && st.partial && tid < BN) kd_next = drow[min(st.k0 + tid, a.S - 1)];
+    };
+    const int my_runs = decltype(sk)::runs_of(w);
     bool have = st.next();
     int k0 = st.k0;
     bool partial = st.partial;
-    if (have) issue(0);
+    if (have) {
+        issue_k(0);
+        issue_v(0);
+        issue_ids();
+    }
 
     for (int n = 0; have; ++n) {
         const int cur = n & 1;
@@ -412,23 +457,51 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dq_bf16_kernel(AttnArgs 
         const int ck0 = k0;
         const bool cpartial = partial;
         have = st.next();
+        bool skip[BN / 32];
+#pragma unroll
+        for (int nb = 0; nb < BN / 32; ++nb) {
+            const int kb0 = ck0 + 32 * nb;
+            skip[nb] = kb0 >= a.S;
+            if (cpartial && bounded && kb0 > qw_hi) skip[nb] = true;
+            if (cpartial && a.window >= 0 && (int64_t)qw_lo - (kb0 + 31) > a.window) skip[nb] = true;
+        }
+        // The tile loads of the next step are spread over this step's first MFMA chains (K tile in
+        // the first 32-row block, V tile in the second), see the dK/dV kernel.
+        int pace = 0;
+        const __bf16 *ksrc = kp, *vsrc = vp;
         if (have) {
             k0 = st.k0;
             partial = st.partial;
-            issue(cur ^ 1);
+            ksrc = kp + (int64_t)k0 * a.k.stride_s;
+            vsrc = vp + (int64_t)k0 * a.v.stride_s;
+            issue_ids();
+            const bool spread = (k0 + BN <= a.S) & !skip[0] & !skip[1];
+            pace = __builtin_amdgcn_readfirstlane(spread ? my_runs : 0);
+            if (!pace) {
+                issue_k(cur ^ 1);
+                issue_v(cur ^ 1);
+            }
         }
+        const uint32_t kdst = lds_addr(Kbuf(cur ^ 1)), vdst = lds_addr(Vbuf(cur ^ 1));
+        const uint32_t ksb = (uint32_t)(a.k.stride_s * 2), vsb = (uint32_t)(a.v.stride_s * 2);
 
 #pragma unroll 1
         for (int nb = 0; nb < BN / 32; ++nb) {
             const int kb0 = ck0 + 32 * nb;
-            if (kb0 >= a.S) continue;
-            if (cpartial && bounded && kb0 > qw_hi) continue;
-            if (cpartial && a.window >= 0 && (int64_t)qw_lo - (kb0 + 31) > a.window) continue;
+            if (nb ? skip[1] : skip[0]) continue;
+            const __bf16* psrc = nb ? vsrc : ksrc;
+            const uint32_t pdst = nb ? vdst : kdst, psb = nb ? vsb : ksb;
+            constexpr int kEvery = (2 * KK) / decltype(sk)::PER;
+            static_assert(kEvery >= 1, "pacing");
+            auto pace_hook = [&](auto idx) {
+                constexpr int i = decltype(idx)::value;
+                if constexpr (i % kEvery == kEvery - 1) sk.template issue_one<i / kEvery>(psrc, pdst, w, pace, psb);
+            };
 
             // S^T = K Q^T and dP^T = V dO^T for 32 kv rows x the wave's 32 q rows (lane owns one q row)
             f32x16 s, dp;
             const uint32_t roff = (uint32_t)(32 * nb * TL::kPitch);
-            rowfrag_gemm2<D, kBPipe, false, true>(lds_addr(Ks) + rbase + roff, qf, s, lds_addr(Vs) + rbase + roff, gf, dp);
+            rowfrag_gemm2<D, kBPipe, false, true>(lds_addr(Ks) + rbase + roff, qf, s, lds_addr(Vs) + rbase + roff, gf, dp, pace_hook);
 
             bf16x8 dsf[2];
             const int qrel = q - kb0 - 4 * hh;                     // d = q - kv = qrel - (8*(v/4) + v%4)

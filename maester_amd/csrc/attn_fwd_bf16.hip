@@ -94,15 +94,16 @@ __global__ __launch_bounds__(kFwdThreads) void attn_fwd_bf16_kernel(AttnArgs a) 
     KvSteps st;
     st.zero = opaque_lane_zero();
     st.walk.init(a.map.kv_indices + mrow * a.T, a.map.kv_num_blocks[mrow], a.map.full_kv_indices + mrow * a.T,
-                 a.map.full_kv_num_blocks[mrow], 1, st.zero);
+                 a.map.full_kv_num_blocks[mrow], 1, false, st.zero);
     st.half = kTile / kFwdBN - 1; st.tile = 0; st.partial = false; st.S = a.S;
     st.q_lo = i * kTile; st.q_hi = i * kTile + kTile - 1;
     st.bounded = bounded; st.window = a.window;
 
     DirectStager<D, BN, kFwdThreads / 64> sk, sv;
-    sk.init(w, lane, a.k.stride_s);
-    sv.init(w, lane, a.v.stride_s);
+    sk.init(w, lane);
+    sv.init(w, lane);
     int64_t kd_next = 0;
+    const int my_runs = decltype(sk)::runs_of(w);
     bool have = st.next();
     int k0 = st.k0;
     bool partial = st.partial;
@@ -118,7 +119,7 @@ __global__ __launch_bounds__(kFwdThreads) void attn_fwd_bf16_kernel(AttnArgs a) 
     {
         lds_ptr Qs = Kbuf(1);
         DirectStager<D, kTile, kFwdThreads / 64> sq;
-        sq.init(w, lane, a.q.stride_s);
+        sq.init(w, lane);
         sq.issue(qp + (int64_t)i * kTile * a.q.stride_s, Qs, w, lane, min(kTile, a.S - i * kTile), a.q.stride_s);
         wait_vmem();
         __syncthreads();
@@ -138,15 +139,6 @@ __global__ __launch_bounds__(kFwdThreads) void attn_fwd_bf16_kernel(AttnArgs a) 
         const int ck0 = k0;
         const bool cpartial = partial;
         have = st.next();
-        if (have) {
-            k0 = st.k0;
-            partial = st.partial;
-            const int rows_valid = min(BN, a.S - k0);
-            sk.issue(kp + (int64_t)k0 * a.k.stride_s, Kbuf(cur ^ 1), w, lane, rows_valid, a.k.stride_s);
-            sv.issue(vp + (int64_t)k0 * a.v.stride_s, Vbuf(cur ^ 1), w, lane, rows_valid, a.v.stride_s);
-            if (HAS_DOC && partial && tid < BN) kd_next = drow[min(k0 + tid, a.S - 1)];
-        }
-
         bool act[2];
 #pragma unroll
         for (int nb = 0; nb < 2; ++nb) {
@@ -156,12 +148,44 @@ __global__ __launch_bounds__(kFwdThreads) void attn_fwd_bf16_kernel(AttnArgs a) 
             if (cpartial && a.window >= 0 && (int64_t)qw_lo - (kb0 + 31) > a.window) on = false;
             act[nb] = on;
         }
-        if (!act[0] && !act[1]) continue;
+        const bool idle = !act[0] & !act[1];
+        // The tile loads of the next step are spread over this step's two MFMA chains (K tile in the
+        // first, V tile in the second), one run every few MFMAs: issued in one burst they fill the
+        // memory pipeline and stall the wave with the matrix cores idle.  A ragged last tile, or a
+        // step without chains, issues them at once.
+        int pace = 0;
+        const __bf16 *ksrc = kp, *vsrc = vp;
+        if (have) {
+            k0 = st.k0;
+            partial = st.partial;
+            ksrc = kp + (int64_t)k0 * a.k.stride_s;
+            vsrc = vp + (int64_t)k0 * a.v.stride_s;
+            if (HAS_DOC && partial && tid < BN) kd_next = drow[min(k0 + tid, a.S - 1)];
+            pace = __builtin_amdgcn_readfirstlane(((k0 + BN <= a.S) & !idle) ? my_runs : 0);
+            if (!pace) {
+                const int rows_valid = min(BN, a.S - k0);
+                sk.issue(ksrc, Kbuf(cur ^ 1), w, lane, rows_valid, a.k.stride_s);
+                sv.issue(vsrc, Vbuf(cur ^ 1), w, lane, rows_valid, a.v.stride_s);
+            }
+        }
+        if (idle) continue;
+        const uint32_t kdst = lds_addr(Kbuf(cur ^ 1)), vdst = lds_addr(Vbuf(cur ^ 1));
+        const uint32_t ksb = (uint32_t)(a.k.stride_s * 2), vsb = (uint32_t)(a.v.stride_s * 2);
+        constexpr int kEvery = (2 * KK) / decltype(sk)::PER;  // both chains have 2*KK MFMAs
+        static_assert(kEvery >= 1 && DB * 4 == 2 * KK, "pacing");
+        auto pace_k = [&](auto idx) {
+            constexpr int i = decltype(idx)::value;
+            if constexpr (i % kEvery == kEvery - 1) sk.template issue_one<i / kEvery>(ksrc, kdst, w, pace, ksb);
+        };
+        auto pace_v = [&](auto idx) {
+            constexpr int i = decltype(idx)::value;
+            if constexpr (i % kEvery == kEvery - 1) sk.template issue_one<i / kEvery>(vsrc, vdst, w, pace, vsb);
+        };
 
         // S^T blocks (kv x q).  Both 32-row blocks are always computed: a block the wave cannot see
         // is masked below, and keeping one straight-line path keeps every accumulator in place.
         f32x16 s[2];
-        rowfrag_gemm<D, 2, kPipe>(lds_addr(Ks) + rbase, qf, s);
+        rowfrag_gemm<D, 2, kPipe>(lds_addr(Ks) + rbase, qf, s, pace_k);
         // scale into log2 units and mask
         float mx = -INFINITY;
         if (cpartial) {
@@ -242,7 +266,7 @@ __global__ __launch_bounds__(kFwdThreads) void attn_fwd_bf16_kernel(AttnArgs a) 
         lsum += rs;
 
         // O^T += V^T P^T
-        trfrag_gemm<D, 4, kPipe>(lds_addr(Vs) + tbase, &pf[0][0], o);
+        trfrag_gemm<D, 4, kPipe>(lds_addr(Vs) + tbase, &pf[0][0], o, pace_v);
     }
 
     // Epilogue: O^T (a lane owns one q row, 4 consecutive d per register group) goes through LDS so

@@ -89,18 +89,24 @@ __device__ __forceinline__ bool map_work(int id, int n_units, int T, int Hkv, in
 // Walks `reps` times over the concatenation of two tile lists (partial tiles, then full tiles) of a
 // tile-map row.  The index of the following entry is always in flight: it is loaded when the current
 // one is handed out and only read (readfirstlane) a whole step later, so the walk never waits on
-// memory.  `zero` must be a per-lane zero the compiler cannot see through (it keeps the load a plain
+// memory.  Walking backward (full tiles from the highest index down, then the partial ones) makes all
+// the workgroups of one document start on the same tile and stay in step, so that they share the
+// stream in L2.  `zero` must be a per-lane zero the compiler cannot see through (it keeps the load a plain
 // per-lane load whose result stays in a vector register until it is needed).
 struct ListWalk {
     const int32_t *pl, *fl;
     int np, n, reps, rep, it;
     int nxt;
+    bool backward;  // walk the concatenation from its last entry to its first
 
-    __device__ __forceinline__ int fetch(int i, int zero) const { return i < np ? pl[i + zero] : fl[i - np + zero]; }
+    __device__ __forceinline__ int fetch(int c, int zero) const {
+        const int i = backward ? n - 1 - c : c;
+        return i < np ? pl[i + zero] : fl[i - np + zero];
+    }
     __device__ __forceinline__ void init(const int32_t* partial_list, int n_partial, const int32_t* full_list, int n_full,
-                                         int repeats, int zero) {
+                                         int repeats, bool reverse, int zero) {
         pl = partial_list; fl = full_list; np = n_partial; n = n_partial + n_full; reps = repeats;
-        rep = 0; it = -1;
+        rep = 0; it = -1; backward = reverse;
         nxt = n ? fetch(0, zero) : 0;
     }
     __device__ __forceinline__ bool advance(int& tile, bool& partial, int zero) {
@@ -110,7 +116,7 @@ struct ListWalk {
             if (++rep == reps) return false;
         }
         tile = __builtin_amdgcn_readfirstlane(nxt);
-        partial = it < np;
+        partial = (backward ? n - 1 - it : it) < np;
         nxt = fetch(it + 1 == n ? 0 : it + 1, zero);
         return true;
     }

@@ -373,7 +373,9 @@ struct DirectStager {
     static_assert(SLOTS % 64 == 0, "tile must be a whole number of wave runs");
     static constexpr int NL = SLOTS / 64;
     static constexpr int PER = (NL + NWAVES - 1) / NWAVES;
-    uint32_t off[PER];  // byte offset of this lane's source from the first row of the tile
+    // (source row << 16 | byte offset inside the row) of this lane for each of its runs: the same for
+    // every tile of this shape, whatever its row stride
+    uint32_t rc[PER];
 
     __device__ __forceinline__ static void slot(int t, int lane, int& row, int& chunk) {
         const int s = t * 64 + lane;
@@ -382,38 +384,35 @@ struct DirectStager {
         if (chunk == TL::kChunks) chunk = 0;
         row = TL::prow(rho);  // prow is its own inverse
     }
-    // run p of wave w; when the runs do not divide evenly the surplus slots of the last round repeat
-    // the last run (same data to the same place), so that every wave issues the same instructions
-    __device__ __forceinline__ static int run_of(int w, int p) { return min(w + p * NWAVES, NL - 1); }
-    __device__ __forceinline__ void init(int w, int lane, int64_t stride) {
+    __device__ __forceinline__ void init(int w, int lane) {
 #pragma unroll
         for (int p = 0; p < PER; ++p) {
             int row, chunk;
-            slot(run_of(w, p), lane, row, chunk);
-            off[p] = (uint32_t)((row * stride + chunk * 8) * 2);
+            slot(w + p * NWAVES, lane, row, chunk);
+            rc[p] = (uint32_t)(row << 16 | chunk * 16);
         }
     }
-    // run P of this wave for a whole tile (all ROWS rows valid)
-    template <int P>
-    __device__ __forceinline__ void issue_one(const __bf16* g, uint32_t tile_addr, int w) const {
-        if constexpr (P < PER) global_to_lds_run(g, off[P], tile_addr + run_of(w, P) * 1024);
+    // number of runs wave w moves per tile
+    __device__ __forceinline__ static int runs_of(int w) { return (NL - w + NWAVES - 1) / NWAVES; }
+    __device__ __forceinline__ uint32_t offset(int p, uint32_t stride_bytes, int last_row) const {
+        return (uint32_t)min((int)(rc[p] >> 16), last_row) * stride_bytes + (rc[p] & 0xffffu);
     }
+    // run P of this wave for a whole tile (all ROWS rows valid), if P < limit (wave-uniform)
+    template <int P>
+    __device__ __forceinline__ void issue_one(const __bf16* g, uint32_t tile_addr, int w, int limit, uint32_t stride_bytes) const {
+        if constexpr (P < PER) {
+            if (P < limit)
+                global_to_lds_run(g, (rc[P] >> 16) * stride_bytes + (rc[P] & 0xffffu), tile_addr + (w + P * NWAVES) * 1024);
+        }
+    }
+    // the whole tile at once; rows at or beyond rows_valid re-read the last valid row
     __device__ __forceinline__ void issue(const __bf16* g, lds_ptr tile, int w, int lane, int rows_valid,
                                           int64_t stride) const {
+        const uint32_t sb = (uint32_t)(stride * 2);
+        const int runs = runs_of(w);
 #pragma unroll
-        for (int p = 0; p < PER; ++p) {
-            const int t = w + p * NWAVES;
-            if (t < NL) {
-                uint32_t o = off[p];
-                if (rows_valid < ROWS) {
-                    int row, chunk;
-                    slot(t, lane, row, chunk);
-                    o = (uint32_t)((min(row, rows_valid - 1) * stride + chunk * 8) * 2);
-                }
-                __builtin_amdgcn_global_load_lds((const MA_GLB void*)((const char*)g + o), (MA_LDS void*)(tile + t * 1024),
-                                                 16, 0, 0);
-            }
-        }
+        for (int p = 0; p < PER; ++p)
+            if (p < runs) global_to_lds_run(g, offset(p, sb, rows_valid - 1), lds_addr(tile) + (w + p * NWAVES) * 1024);
     }
 };
 
