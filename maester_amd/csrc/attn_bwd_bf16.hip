@@ -282,31 +282,38 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dkv_bf16_kernel(AttnArgs
             const unsigned span = (unsigned)(dhi - dlo);
             const bool some = (dhi >= dlo) & kvalid;
             const unsigned t0 = (unsigned)(drel - dlo);
+            // one straight-line body per kind of tile (masked / unmasked): a test inside the element
+            // loop would turn into a branch per element
+            auto elementwise = [&](auto masked_c) {
+                constexpr bool MASKED = decltype(masked_c)::value;
 #pragma unroll
-            for (int g4 = 0; g4 < 4; ++g4) {
-                const int qoff = 32 * mb + 8 * g4 + 4 * hh;
-                const f32x4 l4 = *(MA_LDS f32x4*)(lse2s + qoff);
-                const f32x4 e4 = *(MA_LDS f32x4*)(dls + qoff);
-                i64x2 ida = {0, 0}, idb = {0, 0};
-                if (HAS_DOC && cpartial) {
-                    ida = *(MA_LDS i64x2*)(qdoc + qoff);
-                    idb = *(MA_LDS i64x2*)(qdoc + qoff + 2);
-                }
-                const int64_t ids[4] = {ida[0], ida[1], idb[0], idb[1]};
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int v = 4 * g4 + e;
-                    float p = fast_exp2(s[v] * sl2 - l4[e]);
-                    if (cpartial) {
-                        bool ok = (t0 + (unsigned)(8 * g4 + e) <= span) & some;
-                        if (HAS_DOC) ok = ok & (ids[e] == dock);
-                        p = ok ? p : 0.f;
+                for (int g4 = 0; g4 < 4; ++g4) {
+                    const int qoff = 32 * mb + 8 * g4 + 4 * hh;
+                    const f32x4 l4 = *(MA_LDS f32x4*)(lse2s + qoff);
+                    const f32x4 e4 = *(MA_LDS f32x4*)(dls + qoff);
+                    i64x2 ida = {0, 0}, idb = {0, 0};
+                    if (HAS_DOC && MASKED) {
+                        ida = *(MA_LDS i64x2*)(qdoc + qoff);
+                        idb = *(MA_LDS i64x2*)(qdoc + qoff + 2);
                     }
-                    const float ds = p * (dp[v] - e4[e]);
-                    pf[v >> 3][v & 7] = (__bf16)p;
-                    dsf[v >> 3][v & 7] = (__bf16)ds;
+                    const int64_t ids[4] = {ida[0], ida[1], idb[0], idb[1]};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int v = 4 * g4 + e;
+                        float p = fast_exp2(s[v] * sl2 - l4[e]);
+                        if (MASKED) {
+                            bool ok = (t0 + (unsigned)(8 * g4 + e) <= span) & some;
+                            if (HAS_DOC) ok = ok & (ids[e] == dock);
+                            p = ok ? p : 0.f;
+                        }
+                        const float ds = p * (dp[v] - e4[e]);
+                        pf[v >> 3][v & 7] = (__bf16)p;
+                        dsf[v >> 3][v & 7] = (__bf16)ds;
+                    }
                 }
-            }
+            };
+            if (cpartial) elementwise(std::true_type{});
+            else elementwise(std::false_type{});
             // dV^T += dO^T P and dK^T += Q^T dS  (accumulators stay in AGPRs)
             trfrag_gemm<D, 2, kBPipe, true>(lds_addr(Gs) + tbase + roff, pf, dvacc);
             trfrag_gemm<D, 2, kBPipe, true>(lds_addr(Qs) + tbase + roff, dsf, dkacc);
@@ -509,26 +516,31 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dq_bf16_kernel(AttnArgs 
             const unsigned span = (unsigned)(wlim - dlo);
             const bool some = (wlim >= dlo) & qvalid;
             const unsigned t0 = (unsigned)(qrel - dlo);
+            auto elementwise = [&](auto masked_c) {  // one straight-line body per kind of tile
+                constexpr bool MASKED = decltype(masked_c)::value;
 #pragma unroll
-            for (int g4 = 0; g4 < 4; ++g4) {
-                i64x2 ida = {0, 0}, idb = {0, 0};
-                if (HAS_DOC && cpartial) {
-                    ida = *(MA_LDS i64x2*)(kdoc + 32 * nb + 8 * g4 + 4 * hh);
-                    idb = *(MA_LDS i64x2*)(kdoc + 32 * nb + 8 * g4 + 4 * hh + 2);
-                }
-                const int64_t ids[4] = {ida[0], ida[1], idb[0], idb[1]};
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int v = 4 * g4 + e;
-                    float p = fast_exp2(s[v] * sl2 - lse2);
-                    if (cpartial) {
-                        bool ok = (t0 - (unsigned)(8 * g4 + e) <= span) & some;
-                        if (HAS_DOC) ok = ok & (ids[e] == docq);
-                        p = ok ? p : 0.f;
+                for (int g4 = 0; g4 < 4; ++g4) {
+                    i64x2 ida = {0, 0}, idb = {0, 0};
+                    if (HAS_DOC && MASKED) {
+                        ida = *(MA_LDS i64x2*)(kdoc + 32 * nb + 8 * g4 + 4 * hh);
+                        idb = *(MA_LDS i64x2*)(kdoc + 32 * nb + 8 * g4 + 4 * hh + 2);
                     }
-                    dsf[v >> 3][v & 7] = (__bf16)(p * (dp[v] - delta));
+                    const int64_t ids[4] = {ida[0], ida[1], idb[0], idb[1]};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int v = 4 * g4 + e;
+                        float p = fast_exp2(s[v] * sl2 - lse2);
+                        if (MASKED) {
+                            bool ok = (t0 - (unsigned)(8 * g4 + e) <= span) & some;
+                            if (HAS_DOC) ok = ok & (ids[e] == docq);
+                            p = ok ? p : 0.f;
+                        }
+                        dsf[v >> 3][v & 7] = (__bf16)(p * (dp[v] - delta));
+                    }
                 }
-            }
+            };
+            if (cpartial) elementwise(std::true_type{});
+            else elementwise(std::false_type{});
             // dQ^T += K^T dS^T  (accumulator stays in AGPRs)
             trfrag_gemm<D, 2, kBPipe, true>(lds_addr(Ks) + tbase + roff, dsf, acc);
         }
