@@ -50,6 +50,9 @@ static int check_tensor(const char* who, const char* name, const ma_tensor4* t, 
                     (long long)t->stride_b, (long long)t->stride_s, (long long)t->stride_h, (long long)al);
     if (t->stride_b < 0 || t->stride_s <= 0 || t->stride_h < 0)
         return fail(MA_ERR_BAD_ARG, "%s: strides of %s must be non-negative (stride_s positive)", who, name);
+    // the kernels address the rows of a 128-row tile with 32-bit byte offsets
+    if (t->stride_s * elt >= ((int64_t)1 << 24))
+        return fail(MA_ERR_UNSUPPORTED, "%s: row stride of %s (%lld elements) is 16 MiB or more", who, name, (long long)t->stride_s);
     return MA_OK;
 }
 

@@ -81,31 +81,6 @@ __global__ __launch_bounds__(256) void attn_delta_bf16_kernel(AttnArgs a) {
 // ------------------------------------------------------------------------------------------------
 // dK / dV
 // ------------------------------------------------------------------------------------------------
-// Walks, for each of the G query heads of the kv head, the (partial, then full) q tile lists of one
-// kv tile in steps of kStep q rows, skipping steps no row of the workgroup can see.
-struct QSteps {
-    ListWalk walk;
-    int half, S, k_lo, k_hi, bounded, zero, tile;
-    int64_t window;
-    int q0;
-    bool partial;
-
-    __device__ __forceinline__ int g() const { return walk.rep; }
-    __device__ __forceinline__ bool next() {
-        for (;;) {
-            if (++half == kTile / kStep) {
-                half = 0;
-                if (!walk.advance(tile, partial, zero)) return false;
-            }
-            q0 = tile * kTile + half * kStep;
-            if (q0 >= S) continue;
-            if (partial && bounded && q0 + kStep - 1 < k_lo) continue;
-            if (partial && window >= 0 && (int64_t)q0 - k_hi > window) continue;
-            return true;
-        }
-    }
-};
-
 template <int D, bool HAS_DOC>
 __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dkv_bf16_kernel(AttnArgs a) {
     using TL = Tile<D>;
@@ -169,40 +144,48 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dkv_bf16_kernel(AttnArgs
         for (int v = 0; v < 16; ++v) dkacc[db][v] = dvacc[db][v] = 0.f;
 
     const size_t mrow = (size_t)b * a.T + j;
-    QSteps st;
-    st.zero = opaque_lane_zero();
-    st.walk.init(a.map.q_indices + mrow * a.T, a.map.q_num_blocks[mrow], a.map.full_q_indices + mrow * a.T,
-                 a.map.full_q_num_blocks[mrow], G, true, st.zero);
-    st.half = kTile / kStep - 1; st.tile = 0; st.partial = false; st.S = a.S;
-    st.k_lo = j * kTile; st.k_hi = j * kTile + kTile - 1; st.bounded = bounded; st.window = a.window;
+    // q steps of the kv tile, for each of the G query heads in turn, from the last q tile down (see
+    // ListWalk); limits inside which a 32-row q block of a partial tile can be visible to this wave
+    const bool windowed = a.window >= 0;
+    StepWalk<BM> st;
+    {
+        int lo, hi;
+        visibility_limits(true, j * kTile, j * kTile + kTile - 1, BM, bounded, wlim, windowed, lo, hi);
+        st.init(a.map.q_indices + mrow * a.T, a.map.q_num_blocks[mrow], a.map.full_q_indices + mrow * a.T,
+                a.map.full_q_num_blocks[mrow], G, true, a.S, lo, hi);
+    }
+    int blk_lo, blk_hi;
+    visibility_limits(true, kw_lo, kw_hi, 32, bounded, wlim, windowed, blk_lo, blk_hi);
 
-    DirectStager<D, BM, NW> sq, sg;
+    DirectStager<D, BM, NW> sq;  // the Q and dO tiles have the same shape: one set of slots
     sq.init(w, lane);
-    sg.init(w, lane);
+    const uint32_t qsb = (uint32_t)(a.q.stride_s * 2), gsb = (uint32_t)(a.dout.stride_s * 2);  // row strides in bytes
+    const char* qhead = (const char*)((const __bf16*)a.q.ptr + b * a.q.stride_b);
+    const char* ghead = (const char*)((const __bf16*)a.dout.ptr + b * a.dout.stride_b);
     float lse_next = 0.f, dl_next = 0.f;
     int64_t qd_next = 0;
     // global sources of the step the iterator stands on
-    const __bf16 *qsrc = nullptr, *gsrc = nullptr;
+    const char *qsrc = nullptr, *gsrc = nullptr;
     auto locate = [&]() {
-        const int h = hk * G + st.g();
-        qsrc = (const __bf16*)a.q.ptr + b * a.q.stride_b + h * a.q.stride_h + (int64_t)st.q0 * a.q.stride_s;
-        gsrc = (const __bf16*)a.dout.ptr + b * a.dout.stride_b + h * a.dout.stride_h + (int64_t)st.q0 * a.dout.stride_s;
+        const int h = hk * G + st.walk.rep;
+        qsrc = qhead + (uint64_t)(uint32_t)h * (uint32_t)(a.q.stride_h * 2) + (uint64_t)(uint32_t)st.r0 * qsb;
+        gsrc = ghead + (uint64_t)(uint32_t)h * (uint32_t)(a.dout.stride_h * 2) + (uint64_t)(uint32_t)st.r0 * gsb;
     };
     auto issue_rows = [&]() {  // per-row lse / delta / document id of that step
         if (tid < BM) {
-            const int h = hk * G + st.g();
-            const int qq = min(st.q0 + tid, a.S - 1);
+            const int h = hk * G + st.walk.rep;
+            const int qq = min(st.r0 + tid, a.S - 1);
             const size_t row = ((size_t)b * a.Hq + h) * a.S + qq;
             lse_next = a.lse[row];  // converted to log2 units when it is written to LDS
             dl_next = a.delta[row];
             if (HAS_DOC) qd_next = drow[qq];
         }
     };
-    auto issue_q = [&](int buf) { sq.issue(qsrc, Qbuf(buf), w, lane, min(BM, a.S - st.q0), a.q.stride_s); };
-    auto issue_g = [&](int buf) { sg.issue(gsrc, Gbuf(buf), w, lane, min(BM, a.S - st.q0), a.dout.stride_s); };
+    auto issue_q = [&](int buf) { sq.issue((const __bf16*)qsrc, Qbuf(buf), w, lane, min(BM, a.S - st.r0), a.q.stride_s); };
+    auto issue_g = [&](int buf) { sq.issue((const __bf16*)gsrc, Gbuf(buf), w, lane, min(BM, a.S - st.r0), a.dout.stride_s); };
     const int my_runs = decltype(sq)::runs_of(w);
     bool have = st.next();
-    int q0 = st.q0;
+    int q0 = st.r0;
     bool partial = st.partial;
     if (have) {
         locate();
@@ -234,15 +217,10 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dkv_bf16_kernel(AttnArgs
         // ragged last tile, or a block that is skipped, issues its tile at once.
         bool skip[BM / 32];
 #pragma unroll
-        for (int mb = 0; mb < BM / 32; ++mb) {
-            const int qb0 = cq0 + 32 * mb;
-            skip[mb] = qb0 >= a.S;
-            if (cpartial && bounded && qb0 + 31 < kw_lo) skip[mb] = true;
-            if (cpartial && a.window >= 0 && (int64_t)qb0 - kw_hi > a.window) skip[mb] = true;
-        }
+        for (int mb = 0; mb < BM / 32; ++mb) skip[mb] = !block_visible(cq0 + 32 * mb, a.S, cpartial, blk_lo, blk_hi);
         int pace = 0;
         if (have) {
-            q0 = st.q0;
+            q0 = st.r0;
             partial = st.partial;
             locate();
             issue_rows();
@@ -254,13 +232,12 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dkv_bf16_kernel(AttnArgs
             }
         }
         const uint32_t qdst = lds_addr(Qbuf(cur ^ 1)), gdst = lds_addr(Gbuf(cur ^ 1));
-        const uint32_t qsb = (uint32_t)(a.q.stride_s * 2), gsb = (uint32_t)(a.dout.stride_s * 2);
 
 #pragma unroll 1
         for (int mb = 0; mb < BM / 32; ++mb) {
             const int qb0 = cq0 + 32 * mb;
             if (mb ? skip[1] : skip[0]) continue;
-            const __bf16* psrc = mb ? gsrc : qsrc;
+            const __bf16* psrc = (const __bf16*)(mb ? gsrc : qsrc);
             const uint32_t pdst = mb ? gdst : qdst, psb = mb ? gsb : qsb;
             constexpr int kEvery = (2 * KK) / decltype(sq)::PER;
             static_assert(kEvery >= 1, "pacing");
@@ -335,28 +312,6 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dkv_bf16_kernel(AttnArgs
 // ------------------------------------------------------------------------------------------------
 // dQ
 // ------------------------------------------------------------------------------------------------
-struct KvStepsB {
-    ListWalk walk;
-    int half, S, q_lo, q_hi, bounded, zero, tile;
-    int64_t window;
-    int k0;
-    bool partial;
-
-    __device__ __forceinline__ bool next() {
-        for (;;) {
-            if (++half == kTile / kStep) {
-                half = 0;
-                if (!walk.advance(tile, partial, zero)) return false;
-            }
-            k0 = tile * kTile + half * kStep;
-            if (k0 >= S) continue;
-            if (partial && bounded && k0 > q_hi) continue;
-            if (partial && window >= 0 && (int64_t)q_lo - (k0 + kStep - 1) > window) continue;
-            return true;
-        }
-    }
-};
-
 template <int D, bool HAS_DOC>
 __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dq_bf16_kernel(AttnArgs a) {
     using TL = Tile<D>;
@@ -421,31 +376,34 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dq_bf16_kernel(AttnArgs 
         for (int v = 0; v < 16; ++v) acc[db][v] = 0.f;
 
     const size_t mrow = (size_t)b * a.T + i;
-    KvStepsB st;
-    st.zero = opaque_lane_zero();
-    st.walk.init(a.map.kv_indices + mrow * a.T, a.map.kv_num_blocks[mrow], a.map.full_kv_indices + mrow * a.T,
-                 a.map.full_kv_num_blocks[mrow], 1, false, st.zero);
-    st.half = kTile / kStep - 1; st.tile = 0; st.partial = false; st.S = a.S;
-    st.q_lo = i * kTile; st.q_hi = i * kTile + kTile - 1;
-    st.bounded = bounded; st.window = a.window;
+    const bool windowed = a.window >= 0;
+    StepWalk<BN> st;
+    {
+        int lo, hi;
+        visibility_limits(false, i * kTile, i * kTile + kTile - 1, BN, bounded, wlim, windowed, lo, hi);
+        st.init(a.map.kv_indices + mrow * a.T, a.map.kv_num_blocks[mrow], a.map.full_kv_indices + mrow * a.T,
+                a.map.full_kv_num_blocks[mrow], 1, false, a.S, lo, hi);
+    }
+    int blk_lo, blk_hi;
+    visibility_limits(false, qw_lo, qw_hi, 32, bounded, wlim, windowed, blk_lo, blk_hi);
 
-    DirectStager<D, BN, NW> sk, sv;
+    DirectStager<D, BN, NW> sk;  // the K and V tiles have the same shape: one set of slots
     sk.init(w, lane);
-    sv.init(w, lane);
+    const uint32_t ksb = (uint32_t)(a.k.stride_s * 2), vsb = (uint32_t)(a.v.stride_s * 2);  // row strides in bytes
     int64_t kd_next = 0;
     // the step the iterator stands on
     auto issue_k = [&](int buf) {
-        sk.issue(kp + (int64_t)st.k0 * a.k.stride_s, Kbuf(buf), w, lane, min(BN, a.S - st.k0), a.k.stride_s);
+        sk.issue((const __bf16*)((const char*)kp + (uint64_t)(uint32_t)st.r0 * ksb), Kbuf(buf), w, lane, min(BN, a.S - st.r0), a.k.stride_s);
     };
     auto issue_v = [&](int buf) {
-        sv.issue(vp + (int64_t)st.k0 * a.v.stride_s, Vbuf(buf), w, lane, min(BN, a.S - st.k0), a.v.stride_s);
+        sk.issue((const __bf16*)((const char*)vp + (uint64_t)(uint32_t)st.r0 * vsb), Vbuf(buf), w, lane, min(BN, a.S - st.r0), a.v.stride_s);
     };
     auto issue_ids = [&]() {
-        if (HAS_DOC && st.partial && tid < BN) kd_next = drow[min(st.k0 + tid, a.S - 1)];
+        if (HAS_DOC && st.partial && tid < BN) kd_next = drow[min(st.r0 + tid, a.S - 1)];
     };
     const int my_runs = decltype(sk)::runs_of(w);
     bool have = st.next();
-    int k0 = st.k0;
+    int k0 = st.r0;
     bool partial = st.partial;
     if (have) {
         issue_k(0);
@@ -466,21 +424,16 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dq_bf16_kernel(AttnArgs 
         have = st.next();
         bool skip[BN / 32];
 #pragma unroll
-        for (int nb = 0; nb < BN / 32; ++nb) {
-            const int kb0 = ck0 + 32 * nb;
-            skip[nb] = kb0 >= a.S;
-            if (cpartial && bounded && kb0 > qw_hi) skip[nb] = true;
-            if (cpartial && a.window >= 0 && (int64_t)qw_lo - (kb0 + 31) > a.window) skip[nb] = true;
-        }
+        for (int nb = 0; nb < BN / 32; ++nb) skip[nb] = !block_visible(ck0 + 32 * nb, a.S, cpartial, blk_lo, blk_hi);
         // The tile loads of the next step are spread over this step's first MFMA chains (K tile in
         // the first 32-row block, V tile in the second), see the dK/dV kernel.
         int pace = 0;
         const __bf16 *ksrc = kp, *vsrc = vp;
         if (have) {
-            k0 = st.k0;
+            k0 = st.r0;
             partial = st.partial;
-            ksrc = kp + (int64_t)k0 * a.k.stride_s;
-            vsrc = vp + (int64_t)k0 * a.v.stride_s;
+            ksrc = (const __bf16*)((const char*)kp + (uint64_t)(uint32_t)k0 * ksb);
+            vsrc = (const __bf16*)((const char*)vp + (uint64_t)(uint32_t)k0 * vsb);
             issue_ids();
             const bool spread = (k0 + BN <= a.S) & !skip[0] & !skip[1];
             pace = __builtin_amdgcn_readfirstlane(spread ? my_runs : 0);
@@ -490,7 +443,6 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dq_bf16_kernel(AttnArgs 
             }
         }
         const uint32_t kdst = lds_addr(Kbuf(cur ^ 1)), vdst = lds_addr(Vbuf(cur ^ 1));
-        const uint32_t ksb = (uint32_t)(a.k.stride_s * 2), vsb = (uint32_t)(a.v.stride_s * 2);
 
 #pragma unroll 1
         for (int nb = 0; nb < BN / 32; ++nb) {

@@ -23,30 +23,6 @@ constexpr int kFwdBN = 64;  // kv rows per step
 
 constexpr int kPipe = 4;  // LDS fragment reads kept in flight ahead of the MFMAs
 
-// Walks the (partial, then full) kv tile lists of one q tile in steps of BN rows, skipping the
-// steps no row of the workgroup can see.  All state is workgroup-uniform.
-struct KvSteps {
-    ListWalk walk;
-    int half, S, q_lo, q_hi, bounded, zero, tile;
-    int64_t window;
-    int k0;
-    bool partial;
-
-    __device__ __forceinline__ bool next() {
-        for (;;) {
-            if (++half == kTile / kFwdBN) {
-                half = 0;
-                if (!walk.advance(tile, partial, zero)) return false;
-            }
-            k0 = tile * kTile + half * kFwdBN;
-            if (k0 >= S) continue;
-            if (partial && bounded && k0 > q_hi) continue;
-            if (partial && window >= 0 && (int64_t)q_lo - (k0 + kFwdBN - 1) > window) continue;
-            return true;
-        }
-    }
-};
-
 template <int D, bool HAS_DOC>
 __global__ __launch_bounds__(kFwdThreads) void attn_fwd_bf16_kernel(AttnArgs a) {
     using TL = Tile<D>;
@@ -72,14 +48,26 @@ __global__ __launch_bounds__(kFwdThreads) void attn_fwd_bf16_kernel(AttnArgs a) 
     const bool bounded = a.causal || a.window >= 0;  // kv <= q is part of the predicate
 
     const __bf16* qp = (const __bf16*)a.q.ptr + b * a.q.stride_b + h * a.q.stride_h;
-    const __bf16* kp = (const __bf16*)a.k.ptr + b * a.k.stride_b + hk * a.k.stride_h;
-    const __bf16* vp = (const __bf16*)a.v.ptr + b * a.v.stride_b + hk * a.v.stride_h;
+    const char* kp = (const char*)((const __bf16*)a.k.ptr + b * a.k.stride_b + hk * a.k.stride_h);
+    const char* vp = (const char*)((const __bf16*)a.v.ptr + b * a.v.stride_b + hk * a.v.stride_h);
+    const uint32_t ksb = (uint32_t)(a.k.stride_s * 2), vsb = (uint32_t)(a.v.stride_s * 2);  // row strides in bytes
     const int64_t* drow = HAS_DOC ? a.doc + (size_t)b * a.S : nullptr;
+    const int rbase = TL::row_base(lane), tbase = TL::tr_base(lane);
+
+    // The Q tile comes in through LDS (coalesced 1 KB runs instead of 32 strided rows per load); it
+    // borrows the second K/V buffer pair, which the first step does not use yet.  Its loads go out
+    // first: they depend on nothing but the work item.
+    {
+        DirectStager<D, kTile, kFwdThreads / 64> sq;
+        sq.init(w, lane);
+        sq.issue(qp + (int64_t)i * kTile * a.q.stride_s, Kbuf(1), w, lane, min(kTile, a.S - i * kTile), a.q.stride_s);
+    }
 
     // rows past the end of the sequence read the last valid row; their results are never stored
     const int qc = min(q, a.S - 1);
     const int64_t docq = HAS_DOC ? drow[qc] : 0;
-    const int wlim = a.window >= 0 ? (int)min(a.window, (int64_t)0x3fffffff) : 0x7fffffff;
+    const bool windowed = a.window >= 0;
+    const int wlim = windowed ? (int)min(a.window, (int64_t)0x3fffffff) : 0x7fffffff;
 
     f32x16 o[DB];
 #pragma unroll
@@ -88,39 +76,36 @@ __global__ __launch_bounds__(kFwdThreads) void attn_fwd_bf16_kernel(AttnArgs a) 
         for (int v = 0; v < 16; ++v) o[db][v] = 0.f;
     float m = -INFINITY, lsum = 0.f;
     const float sl2 = a.scale * kLog2e;
-    const int rbase = TL::row_base(lane), tbase = TL::tr_base(lane);
 
+    // kv steps of the workgroup's tile row, and the limits inside which a 32-row kv block of a
+    // partial tile can be visible to this wave
     const size_t mrow = (size_t)b * a.T + i;
-    KvSteps st;
-    st.zero = opaque_lane_zero();
-    st.walk.init(a.map.kv_indices + mrow * a.T, a.map.kv_num_blocks[mrow], a.map.full_kv_indices + mrow * a.T,
-                 a.map.full_kv_num_blocks[mrow], 1, false, st.zero);
-    st.half = kTile / kFwdBN - 1; st.tile = 0; st.partial = false; st.S = a.S;
-    st.q_lo = i * kTile; st.q_hi = i * kTile + kTile - 1;
-    st.bounded = bounded; st.window = a.window;
+    StepWalk<BN> st;
+    {
+        int lo, hi;
+        visibility_limits(false, i * kTile, i * kTile + kTile - 1, BN, bounded, wlim, windowed, lo, hi);
+        st.init(a.map.kv_indices + mrow * a.T, a.map.kv_num_blocks[mrow], a.map.full_kv_indices + mrow * a.T,
+                a.map.full_kv_num_blocks[mrow], 1, false, a.S, lo, hi);
+    }
+    int blk_lo, blk_hi;
+    visibility_limits(false, qw_lo, qw_hi, 32, bounded, wlim, windowed, blk_lo, blk_hi);
 
-    DirectStager<D, BN, kFwdThreads / 64> sk, sv;
+    DirectStager<D, BN, kFwdThreads / 64> sk;  // the K and V tiles have the same shape: one set of slots
     sk.init(w, lane);
-    sv.init(w, lane);
     int64_t kd_next = 0;
     const int my_runs = decltype(sk)::runs_of(w);
     bool have = st.next();
-    int k0 = st.k0;
+    int k0 = st.r0;
     bool partial = st.partial;
     if (have) {
         const int rows_valid = min(BN, a.S - k0);
-        sk.issue(kp + (int64_t)k0 * a.k.stride_s, Kbuf(0), w, lane, rows_valid, a.k.stride_s);
-        sv.issue(vp + (int64_t)k0 * a.v.stride_s, Vbuf(0), w, lane, rows_valid, a.v.stride_s);
+        sk.issue((const __bf16*)(kp + (uint64_t)(uint32_t)k0 * ksb), Kbuf(0), w, lane, rows_valid, a.k.stride_s);
+        sk.issue((const __bf16*)(vp + (uint64_t)(uint32_t)k0 * vsb), Vbuf(0), w, lane, rows_valid, a.v.stride_s);
         if (HAS_DOC && partial && tid < BN) kd_next = drow[min(k0 + tid, a.S - 1)];
     }
-    // The Q tile comes in through LDS too (coalesced 1 KB runs instead of 32 strided rows per
-    // load); it borrows the second K/V buffer pair, which the first step does not use yet.
     bf16x8 qf[KK];
     {
         lds_ptr Qs = Kbuf(1);
-        DirectStager<D, kTile, kFwdThreads / 64> sq;
-        sq.init(w, lane);
-        sq.issue(qp + (int64_t)i * kTile * a.q.stride_s, Qs, w, lane, min(kTile, a.S - i * kTile), a.q.stride_s);
         wait_vmem();
         __syncthreads();
 #pragma unroll
@@ -141,45 +126,38 @@ __global__ __launch_bounds__(kFwdThreads) void attn_fwd_bf16_kernel(AttnArgs a) 
         have = st.next();
         bool act[2];
 #pragma unroll
-        for (int nb = 0; nb < 2; ++nb) {
-            const int kb0 = ck0 + 32 * nb;
-            bool on = kb0 < a.S;
-            if (cpartial && bounded && kb0 > qw_hi) on = false;
-            if (cpartial && a.window >= 0 && (int64_t)qw_lo - (kb0 + 31) > a.window) on = false;
-            act[nb] = on;
-        }
+        for (int nb = 0; nb < 2; ++nb) act[nb] = block_visible(ck0 + 32 * nb, a.S, cpartial, blk_lo, blk_hi);
         const bool idle = !act[0] & !act[1];
         // The tile loads of the next step are spread over this step's two MFMA chains (K tile in the
         // first, V tile in the second), one run every few MFMAs: issued in one burst they fill the
         // memory pipeline and stall the wave with the matrix cores idle.  A ragged last tile, or a
         // step without chains, issues them at once.
         int pace = 0;
-        const __bf16 *ksrc = kp, *vsrc = vp;
+        const char *ksrc = kp, *vsrc = vp;
         if (have) {
-            k0 = st.k0;
+            k0 = st.r0;
             partial = st.partial;
-            ksrc = kp + (int64_t)k0 * a.k.stride_s;
-            vsrc = vp + (int64_t)k0 * a.v.stride_s;
+            ksrc = kp + (uint64_t)(uint32_t)k0 * ksb;
+            vsrc = vp + (uint64_t)(uint32_t)k0 * vsb;
             if (HAS_DOC && partial && tid < BN) kd_next = drow[min(k0 + tid, a.S - 1)];
             pace = __builtin_amdgcn_readfirstlane(((k0 + BN <= a.S) & !idle) ? my_runs : 0);
             if (!pace) {
                 const int rows_valid = min(BN, a.S - k0);
-                sk.issue(ksrc, Kbuf(cur ^ 1), w, lane, rows_valid, a.k.stride_s);
-                sv.issue(vsrc, Vbuf(cur ^ 1), w, lane, rows_valid, a.v.stride_s);
+                sk.issue((const __bf16*)ksrc, Kbuf(cur ^ 1), w, lane, rows_valid, a.k.stride_s);
+                sk.issue((const __bf16*)vsrc, Vbuf(cur ^ 1), w, lane, rows_valid, a.v.stride_s);
             }
         }
         if (idle) continue;
         const uint32_t kdst = lds_addr(Kbuf(cur ^ 1)), vdst = lds_addr(Vbuf(cur ^ 1));
-        const uint32_t ksb = (uint32_t)(a.k.stride_s * 2), vsb = (uint32_t)(a.v.stride_s * 2);
         constexpr int kEvery = (2 * KK) / decltype(sk)::PER;  // both chains have 2*KK MFMAs
         static_assert(kEvery >= 1 && DB * 4 == 2 * KK, "pacing");
         auto pace_k = [&](auto idx) {
             constexpr int i = decltype(idx)::value;
-            if constexpr (i % kEvery == kEvery - 1) sk.template issue_one<i / kEvery>(ksrc, kdst, w, pace, ksb);
+            if constexpr (i % kEvery == kEvery - 1) sk.template issue_one<i / kEvery>((const __bf16*)ksrc, kdst, w, pace, ksb);
         };
         auto pace_v = [&](auto idx) {
             constexpr int i = decltype(idx)::value;
-            if constexpr (i % kEvery == kEvery - 1) sk.template issue_one<i / kEvery>(vsrc, vdst, w, pace, vsb);
+            if constexpr (i % kEvery == kEvery - 1) sk.template issue_one<i / kEvery>((const __bf16*)vsrc, vdst, w, pace, vsb);
         };
 
         // S^T blocks (kv x q).  Both 32-row blocks are always computed: a block the wave cannot see
@@ -266,7 +244,7 @@ __global__ __launch_bounds__(kFwdThreads) void attn_fwd_bf16_kernel(AttnArgs a) 
         lsum += rs;
 
         // O^T += V^T P^T
-        trfrag_gemm<D, 4, kPipe>(lds_addr(Vs) + tbase, &pf[0][0], o, pace_v);
+        trfrag_gemm<D, 4, 6>(lds_addr(Vs) + tbase, &pf[0][0], o, pace_v);
     }
 
     // Epilogue: O^T (a lane owns one q row, 4 consecutive d per register group) goes through LDS so

@@ -121,6 +121,57 @@ struct ListWalk {
         return true;
     }
 };
+// Steps of STEP rows over a ListWalk of 128-row tiles.  A step is handed out when one of its rows
+// can be visible to the workgroup: it starts inside the sequence and, for a partial tile, inside
+// [vis_lo, vis_hi] -- the causal / window bounds of the workgroup's own rows folded into two 32-bit
+// limits by the caller (full tiles are visible throughout by construction).
+constexpr int kNoLimitLo = -0x40000000, kNoLimitHi = 0x7fffffff;
+template <int STEP>
+struct StepWalk {
+    ListWalk walk;
+    int zero, half, tile, S, vis_lo, vis_hi;
+    int r0;  // first row of the step
+    bool partial;
+
+    __device__ __forceinline__ void init(const int32_t* partial_list, int n_partial, const int32_t* full_list, int n_full,
+                                         int repeats, bool reverse, int seq_len, int lo, int hi) {
+        zero = opaque_lane_zero_();
+        walk.init(partial_list, n_partial, full_list, n_full, repeats, reverse, zero);
+        half = kTile / STEP - 1; tile = 0; partial = false; S = seq_len; vis_lo = lo; vis_hi = hi; r0 = 0;
+    }
+    __device__ __forceinline__ static int opaque_lane_zero_() {
+        int z;
+        asm volatile("v_mov_b32 %0, 0" : "=v"(z));
+        return z;
+    }
+    __device__ __forceinline__ bool next() {
+        for (;;) {
+            if (++half == kTile / STEP) {
+                half = 0;
+                if (!walk.advance(tile, partial, zero)) return false;
+            }
+            r0 = tile * kTile + half * STEP;
+            if ((r0 < S) & (!partial | ((r0 >= vis_lo) & (r0 <= vis_hi)))) return true;
+        }
+    }
+};
+// the same test for a block of rows starting at r0 (bounds of the wave's own rows)
+__device__ __forceinline__ bool block_visible(int r0, int S, bool partial, int lo, int hi) {
+    return (r0 < S) & (!partial | ((r0 >= lo) & (r0 <= hi)));
+}
+// Visibility limits for a walk over kv rows by query rows [q_lo, q_hi] (kv_side = false) or over
+// query rows by kv rows [k_lo, k_hi] (kv_side = true), for steps/blocks of `rows` rows.
+__device__ __forceinline__ void visibility_limits(bool kv_side, int own_lo, int own_hi, int rows, bool bounded, int wlim,
+                                                  bool windowed, int& lo, int& hi) {
+    if (!kv_side) {  // kv block [r0, r0+rows): needs r0 <= q_hi (kv <= q) and r0 + rows - 1 >= q_lo - window
+        hi = bounded ? own_hi : kNoLimitHi;
+        lo = windowed ? own_lo - wlim - (rows - 1) : kNoLimitLo;
+    } else {         // q block [r0, r0+rows): needs r0 + rows - 1 >= k_lo (q >= kv) and r0 <= k_hi + window
+        lo = bounded ? own_lo - (rows - 1) : kNoLimitLo;
+        hi = windowed ? own_hi + wlim : kNoLimitHi;
+    }
+}
+
 __device__ __forceinline__ int opaque_lane_zero() {
     int z;
     asm volatile("v_mov_b32 %0, 0" : "=v"(z));
