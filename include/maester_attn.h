@@ -37,6 +37,7 @@ extern "C" {
 #define MA_DTYPE_BF16 1
 
 #define MA_TILE 128 /* BlockMask tile edge (torch _DEFAULT_SPARSE_BLOCK_SIZE) */
+#define MA_DOC_BLOCK 32 /* rows per entry of ma_tile_map.block_doc_range */
 
 /* Library version (major*10000 + minor*100 + patch). */
 int ma_version(void);
@@ -66,6 +67,11 @@ typedef struct ma_tile_map {
      * (natural order). */
     int32_t* q_tile_order;       /* [B*T] */
     int32_t* kv_tile_order;      /* [B*T] */
+    /* Document-id range (min, max) of every block of MA_DOC_BLOCK consecutive rows (not part of
+     * BlockMask either): inside a partial tile the kernels skip the 32x32 sub-blocks whose q rows
+     * and kv rows have disjoint id ranges -- no pair of them can share a document.  May be NULL, and
+     * is ignored when document_ids is NULL (then nothing is skipped on that ground). */
+    int64_t* block_doc_range;    /* [B, 2 * ceil(S / 64), 2]: blocks past the end repeat the last row */
 } ma_tile_map;
 
 /* ---- block-sparse tile map --------------------------------------------------------------------

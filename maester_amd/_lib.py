@@ -20,6 +20,7 @@ MA_ERR_LAUNCH = -3
 MA_DTYPE_F32 = 0
 MA_DTYPE_BF16 = 1
 MA_TILE = 128
+MA_DOC_BLOCK = 32
 MA_BWD_DELTA, MA_BWD_DKV, MA_BWD_DQ, MA_BWD_ALL = 1, 2, 4, 7
 
 EXPORTS = (
@@ -36,7 +37,8 @@ class MaTensor4(Structure):
 class MaTileMap(Structure):
     _fields_ = [(n, c_void_p) for n in (
         "kv_num_blocks", "kv_indices", "full_kv_num_blocks", "full_kv_indices",
-        "q_num_blocks", "q_indices", "full_q_num_blocks", "full_q_indices", "q_tile_order", "kv_tile_order")]
+        "q_num_blocks", "q_indices", "full_q_num_blocks", "full_q_indices", "q_tile_order", "kv_tile_order",
+        "block_doc_range")]
 
 
 class MaesterAttnError(RuntimeError):

@@ -156,6 +156,14 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dkv_bf16_kernel(AttnArgs
     }
     int blk_lo, blk_hi;
     visibility_limits(true, kw_lo, kw_hi, 32, bounded, wlim, windowed, blk_lo, blk_hi);
+    // document-id ranges: of the wave's own kv rows now, of the two q blocks of a step at each step
+    const bool use_rng = HAS_DOC && a.map.block_doc_range != nullptr;
+    const int64_t* rng_row = use_rng ? a.map.block_doc_range + (size_t)b * (2 * ((a.S + 63) / 64)) * 2 : nullptr;
+    DocRange own;
+    if (use_rng) {
+        own.load(rng_row + (size_t)(min(kw_lo, a.S - 1) / MA_DOC_BLOCK) * 2);
+        own.ready();
+    }
 
     DirectStager<D, BM, NW> sq;  // the Q and dO tiles have the same shape: one set of slots
     sq.init(w, lane);
@@ -200,6 +208,8 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dkv_bf16_kernel(AttnArgs
         MA_LDS float* lse2s = Lbuf(cur);
         MA_LDS float* dls = Ebuf(cur);
         MA_LDS int64_t* qdoc = Dbuf(cur);
+        DocRange2 rng;
+        if (use_rng && partial) rng.load(rng_row + (size_t)(q0 / MA_DOC_BLOCK) * 2);
         if (tid < BM) {
             lse2s[tid] = lse_next * kLog2e;
             dls[tid] = dl_next;
@@ -218,6 +228,11 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dkv_bf16_kernel(AttnArgs
         bool skip[BM / 32];
 #pragma unroll
         for (int mb = 0; mb < BM / 32; ++mb) skip[mb] = !block_visible(cq0 + 32 * mb, a.S, cpartial, blk_lo, blk_hi);
+        if (use_rng && cpartial) {  // no q row of the block shares a document with the wave's kv rows
+            rng.ready();
+#pragma unroll
+            for (int mb = 0; mb < BM / 32; ++mb) skip[mb] |= !rng.meets(mb, own.lo(), own.hi());
+        }
         int pace = 0;
         if (have) {
             q0 = st.r0;
@@ -386,6 +401,14 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dq_bf16_kernel(AttnArgs 
     }
     int blk_lo, blk_hi;
     visibility_limits(false, qw_lo, qw_hi, 32, bounded, wlim, windowed, blk_lo, blk_hi);
+    // document-id ranges: of the wave's own q rows now, of the two kv blocks of a step at each step
+    const bool use_rng = HAS_DOC && a.map.block_doc_range != nullptr;
+    const int64_t* rng_row = use_rng ? a.map.block_doc_range + (size_t)b * (2 * ((a.S + 63) / 64)) * 2 : nullptr;
+    DocRange own;
+    if (use_rng) {
+        own.load(rng_row + (size_t)(min(qw_lo, a.S - 1) / MA_DOC_BLOCK) * 2);
+        own.ready();
+    }
 
     DirectStager<D, BN, NW> sk;  // the K and V tiles have the same shape: one set of slots
     sk.init(w, lane);
@@ -415,6 +438,8 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dq_bf16_kernel(AttnArgs 
         const int cur = n & 1;
         const lds_ptr Ks = Kbuf(cur), Vs = Vbuf(cur);
         MA_LDS int64_t* kdoc = Dbuf(cur);
+        DocRange2 rng;
+        if (use_rng && partial) rng.load(rng_row + (size_t)(k0 / MA_DOC_BLOCK) * 2);
         if (HAS_DOC && partial && tid < BN) kdoc[tid] = kd_next;
         wait_vmem();
         __syncthreads();
@@ -425,6 +450,11 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dq_bf16_kernel(AttnArgs 
         bool skip[BN / 32];
 #pragma unroll
         for (int nb = 0; nb < BN / 32; ++nb) skip[nb] = !block_visible(ck0 + 32 * nb, a.S, cpartial, blk_lo, blk_hi);
+        if (use_rng && cpartial) {  // no kv row of the block shares a document with the wave's q rows
+            rng.ready();
+#pragma unroll
+            for (int nb = 0; nb < BN / 32; ++nb) skip[nb] |= !rng.meets(nb, own.lo(), own.hi());
+        }
         // The tile loads of the next step are spread over this step's first MFMA chains (K tile in
         // the first 32-row block, V tile in the second), see the dK/dV kernel.
         int pace = 0;

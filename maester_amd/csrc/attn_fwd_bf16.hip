@@ -89,6 +89,14 @@ __global__ __launch_bounds__(kFwdThreads) void attn_fwd_bf16_kernel(AttnArgs a) 
     }
     int blk_lo, blk_hi;
     visibility_limits(false, qw_lo, qw_hi, 32, bounded, wlim, windowed, blk_lo, blk_hi);
+    // document-id ranges: of the wave's own q rows now, of the two kv blocks of a step at each step
+    const bool use_rng = HAS_DOC && a.map.block_doc_range != nullptr;
+    const int64_t* rng_row = use_rng ? a.map.block_doc_range + (size_t)b * (2 * ((a.S + 63) / 64)) * 2 : nullptr;
+    DocRange own;
+    if (use_rng) {
+        own.load(rng_row + (size_t)(min(qw_lo, a.S - 1) / MA_DOC_BLOCK) * 2);
+        own.ready();
+    }
 
     DirectStager<D, BN, kFwdThreads / 64> sk;  // the K and V tiles have the same shape: one set of slots
     sk.init(w, lane);
@@ -117,6 +125,8 @@ __global__ __launch_bounds__(kFwdThreads) void attn_fwd_bf16_kernel(AttnArgs a) 
         const int cur = n & 1;
         lds_ptr Ks = Kbuf(cur), Vs = Vbuf(cur);
         MA_LDS int64_t* kdoc = Dbuf(cur);
+        DocRange2 rng;
+        if (use_rng && partial) rng.load(rng_row + (size_t)(k0 / MA_DOC_BLOCK) * 2);
         if (HAS_DOC && partial && tid < BN) kdoc[tid] = kd_next;
         wait_vmem();       // this wave's share of the current tiles has landed ...
         __syncthreads();   // ... and so has everyone's; all waves are also done with the other buffers
@@ -127,6 +137,11 @@ __global__ __launch_bounds__(kFwdThreads) void attn_fwd_bf16_kernel(AttnArgs a) 
         bool act[2];
 #pragma unroll
         for (int nb = 0; nb < 2; ++nb) act[nb] = block_visible(ck0 + 32 * nb, a.S, cpartial, blk_lo, blk_hi);
+        if (use_rng && cpartial) {  // no kv row of the block shares a document with the wave's q rows
+            rng.ready();
+#pragma unroll
+            for (int nb = 0; nb < 2; ++nb) act[nb] &= rng.meets(nb, own.lo(), own.hi());
+        }
         const bool idle = !act[0] & !act[1];
         // The tile loads of the next step are spread over this step's two MFMA chains (K tile in the
         // first, V tile in the second), one run every few MFMAs: issued in one burst they fill the

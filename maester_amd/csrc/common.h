@@ -172,6 +172,28 @@ __device__ __forceinline__ void visibility_limits(bool kv_side, int own_lo, int 
     }
 }
 
+// ---- document-id ranges of 32-row blocks (ma_tile_map.block_doc_range) ---------------------------
+// Fetched with scalar loads (plain reads through the scalar cache): the data is workgroup-uniform.
+// A load is issued early (load_*) and waited for just before its first use (ready()).
+typedef int i32x4_t __attribute__((ext_vector_type(4)));
+typedef int i32x8_t __attribute__((ext_vector_type(8)));
+struct DocRange {      // one block
+    i32x4_t raw;
+    __device__ __forceinline__ void load(const int64_t* entry) { asm volatile("s_load_dwordx4 %0, %1, 0x0" : "=s"(raw) : "s"(entry)); }
+    __device__ __forceinline__ void ready() { asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(raw)); }
+    __device__ __forceinline__ int64_t lo() const { return (int64_t)(((uint64_t)(uint32_t)raw[1] << 32) | (uint32_t)raw[0]); }
+    __device__ __forceinline__ int64_t hi() const { return (int64_t)(((uint64_t)(uint32_t)raw[3] << 32) | (uint32_t)raw[2]); }
+};
+struct DocRange2 {     // two consecutive blocks (one 64-row step)
+    i32x8_t raw;
+    __device__ __forceinline__ void load(const int64_t* entry) { asm volatile("s_load_dwordx8 %0, %1, 0x0" : "=s"(raw) : "s"(entry)); }
+    __device__ __forceinline__ void ready() { asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(raw)); }
+    __device__ __forceinline__ int64_t lo(int k) const { return (int64_t)(((uint64_t)(uint32_t)raw[4 * k + 1] << 32) | (uint32_t)raw[4 * k]); }
+    __device__ __forceinline__ int64_t hi(int k) const { return (int64_t)(((uint64_t)(uint32_t)raw[4 * k + 3] << 32) | (uint32_t)raw[4 * k + 2]); }
+    // can block k share a document with rows whose ids span [own_lo, own_hi]?
+    __device__ __forceinline__ bool meets(int k, int64_t own_lo, int64_t own_hi) const { return (lo(k) <= own_hi) & (hi(k) >= own_lo); }
+};
+
 __device__ __forceinline__ int opaque_lane_zero() {
     int z;
     asm volatile("v_mov_b32 %0, 0" : "=v"(z));

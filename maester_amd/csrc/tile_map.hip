@@ -114,6 +114,26 @@ __global__ __launch_bounds__(1024) void schedule_kernel(int N, ma_tile_map out) 
     }
 }
 
+// (min, max) document id of every block of MA_DOC_BLOCK rows; one half-wave per block.
+__global__ __launch_bounds__(256) void block_ranges_kernel(const int64_t* __restrict__ doc, int B, int S, int NB,
+                                                           int64_t* __restrict__ out) {
+    const int blk = blockIdx.x * 8 + threadIdx.x / MA_DOC_BLOCK;  // 8 blocks per workgroup
+    const int l = threadIdx.x % MA_DOC_BLOCK;
+    if (blk >= B * NB) return;
+    const int b = blk / NB, r0 = (blk % NB) * MA_DOC_BLOCK;
+    const int row = min(r0 + l, S - 1);  // rows past the end repeat the last one
+    int64_t lo = doc[(size_t)b * S + row], hi = lo;
+    for (int off = MA_DOC_BLOCK / 2; off > 0; off >>= 1) {
+        const int64_t olo = __shfl_xor(lo, off, MA_DOC_BLOCK), ohi = __shfl_xor(hi, off, MA_DOC_BLOCK);
+        lo = min(lo, olo);
+        hi = max(hi, ohi);
+    }
+    if (l == 0) {
+        out[(size_t)blk * 2] = lo;
+        out[(size_t)blk * 2 + 1] = hi;
+    }
+}
+
 int launch_tile_map(const int64_t* doc, int B, int S, int causal, int64_t window, const ma_tile_map& out,
                     void* ws, hipStream_t st) {
     const int T = (S + kTile - 1) / kTile;
@@ -123,7 +143,14 @@ int launch_tile_map(const int64_t* doc, int B, int S, int causal, int64_t window
     if (rc) return rc;
     hipLaunchKernelGGL(order_lists_kernel, dim3(T, B, 4), dim3(64), 0, st, cls, T, out);
     rc = check_launch("order_lists_kernel");
-    if (rc || (!out.q_tile_order && !out.kv_tile_order)) return rc;
+    if (rc) return rc;
+    if (doc && out.block_doc_range) {
+        const int NB = 2 * ((S + 63) / 64);
+        hipLaunchKernelGGL(block_ranges_kernel, dim3((B * NB + 7) / 8), dim3(256), 0, st, doc, B, S, NB, out.block_doc_range);
+        rc = check_launch("block_ranges_kernel");
+        if (rc) return rc;
+    }
+    if (!out.q_tile_order && !out.kv_tile_order) return rc;
     hipLaunchKernelGGL(schedule_kernel, dim3(2), dim3(1024), 0, st, B * T, out);
     return check_launch("schedule_kernel");
 }

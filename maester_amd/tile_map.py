@@ -36,6 +36,8 @@ class TileMap:
     # launch schedules (not part of BlockMask): tile rows b*T+i by descending work, int32 [B*T]
     q_tile_order: torch.Tensor | None = None
     kv_tile_order: torch.Tensor | None = None
+    # (min, max) document id of every 32-row block, int64 [B, 2*ceil(S/64), 2]; None without document ids
+    block_doc_range: torch.Tensor | None = None
 
     NAMES = ("kv_num_blocks", "kv_indices", "full_kv_num_blocks", "full_kv_indices",
              "q_num_blocks", "q_indices", "full_q_num_blocks", "full_q_indices")
@@ -45,7 +47,7 @@ class TileMap:
 
     def c_struct(self) -> _lib.MaTileMap:
         ptrs = [c_void_p(getattr(self, n).data_ptr()) for n in self.NAMES]
-        ptrs += [None if t is None else c_void_p(t.data_ptr()) for t in (self.q_tile_order, self.kv_tile_order)]
+        ptrs += [None if t is None else c_void_p(t.data_ptr()) for t in (self.q_tile_order, self.kv_tile_order, self.block_doc_range)]
         return _lib.MaTileMap(*ptrs)
 
     @property
@@ -81,6 +83,9 @@ def build_tile_map(document_ids: torch.Tensor | None, batch_size: int, seq_len: 
     tm = TileMap(nums[0], idxs[0], nums[1], idxs[1], nums[2], idxs[2], nums[3], idxs[3],
                  seq_len=seq_len, causal=bool(causal), window=sliding_window, q_tile_order=order[0],
                  kv_tile_order=order[1])
+    if document_ids is not None:
+        nblk = 2 * ((seq_len + 63) // 64)   # two 32-row blocks per 64-row step, the last step padded
+        tm.block_doc_range = torch.empty(batch_size, nblk, 2, dtype=torch.int64, device=device)
     ws_bytes = L.ma_tile_map_workspace_bytes(batch_size, seq_len)
     ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=device)
     cs = tm.c_struct()

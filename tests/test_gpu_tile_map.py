@@ -92,3 +92,18 @@ def test_launch_schedule_orders(gpu, name, S):
     assert sorted(q_order.tolist()) == list(range(sp.B * T)) and sorted(kv_order.tolist()) == list(range(sp.B * T))
     assert np.array_equal(q_order, _expected_order(d["kv_num_blocks"], d["full_kv_num_blocks"]))
     assert np.array_equal(kv_order, _expected_order(d["q_num_blocks"], d["full_q_num_blocks"]))
+
+
+@pytest.mark.parametrize("name,S", [("c2", 8192), ("c1", 2048), ("c2", 1000), ("c2", 970)])
+def test_block_document_ranges(gpu, name, S):
+    """(min, max) document id per 32-row block, two blocks per 64-row step, tail rows repeat the last id."""
+    wl = workloads.make(name, S=S, pad_tail=17)
+    sp = wl.spec
+    tm = build_tile_map(wl.document_ids.to(gpu), sp.B, sp.S, True, sp.window)
+    got = tm.block_doc_range.cpu().numpy()
+    nblk = 2 * ((S + 63) // 64)
+    assert got.shape == (sp.B, nblk, 2)
+    ids = wl.document_ids.numpy()
+    padded = np.concatenate([ids, np.repeat(ids[:, -1:], nblk * 32 - S, axis=1)], axis=1).reshape(sp.B, nblk, 32)
+    assert np.array_equal(got[..., 0], padded.min(-1)) and np.array_equal(got[..., 1], padded.max(-1))
+    assert build_tile_map(None, sp.B, sp.S, True, None, device=gpu).block_doc_range is None
