@@ -4,14 +4,16 @@
 // (torch/_higher_order_ops/flex_attention.py:825-993):
 //   delta = rowsum(O * dO);  P = exp(S - lse);  dV = P^T dO;  dS = P * (dO V^T - delta);
 //   dQ = scale * dS K;  dK = scale * dS^T Q;  dK/dV summed over the query heads of a kv head.
-// Three kernels, no atomics anywhere (results are run-to-run identical):
-//   1. delta                      -- one pass over O and dO;
+// Two kernels (three when delta is asked for on its own), no atomics anywhere (results are
+// run-to-run identical):
+//   1. dQ: the forward's decomposition (128-row q tile per workgroup, 32 rows per wave, K/V
+//      64 rows per step through LDS), recomputing S^T and dP^T; it also computes delta for its own
+//      rows (it holds their dO fragments anyway) and writes it out for the second kernel;
 //   2. dK/dV: one workgroup owns a 128-row kv tile of one (batch row, kv head), wave w its rows
 //      32w..32w+31 (K, V fragments and the fp32 dK^T/dV^T accumulators in registers); it walks
 //      the q-side lists of the tile map for each of the G query heads, 64 q rows per step
 //      through LDS, recomputing S and dP;
-//   3. dQ: the forward's decomposition (128-row q tile per workgroup, 32 rows per wave, K/V
-//      64 rows per step through LDS), recomputing S^T and dP^T.
+//   (delta alone: one pass over O and dO.)
 // All products are arranged so that P and dS stay in registers between the two MFMAs that
 // produce and consume them (see mfma.h).
 #include "common.h"
@@ -363,17 +365,30 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dq_bf16_kernel(AttnArgs 
     const int wlim = a.window >= 0 ? (int)min(a.window, (int64_t)0x3fffffff) : 0x7fffffff;
     const size_t rowi = ((size_t)b * a.Hq + h) * a.S + qc;
     const float lse2 = a.lse[rowi] * kLog2e;
-    const float delta = a.delta[rowi];
+    // delta = rowsum(O * dO) of the wave's rows: computed here when the caller asked for that stage
+    // together with this one (the dO rows are on hand anyway), read back otherwise
+    const bool own_delta = (a.stages & MA_BWD_DELTA) != 0;
+    float delta = own_delta ? 0.f : a.delta[rowi];
 
     // Q and dO rows of the workgroup come in through LDS (coalesced) and stay in registers (AGPRs)
     bf16x8 qf[KK], gf[KK];
     {
-        DirectStager<D, kTile, NW> sq, sg;
+        DirectStager<D, kTile, NW> sq;
         sq.init(w, lane);
-        sg.init(w, lane);
         const int rows_valid = min(kTile, a.S - i * kTile);
         sq.issue(qp + (int64_t)i * kTile * a.q.stride_s, Kbuf(0), w, lane, rows_valid, a.q.stride_s);
-        sg.issue(gp + (int64_t)i * kTile * a.dout.stride_s, Kbuf(1), w, lane, rows_valid, a.dout.stride_s);
+        sq.issue(gp + (int64_t)i * kTile * a.dout.stride_s, Kbuf(1), w, lane, rows_valid, a.dout.stride_s);
+        // the wave's O rows go straight to registers, whole rows per load (coalesced); they meet the
+        // dO rows, read back from the LDS tile in the same row-major order, in delta's dot products
+        constexpr int CH = D / 8, RPI = 64 / CH, NIT = 32 / RPI;  // 16-byte chunks per row, rows per load, loads
+        const int orow = lane / CH, oc = lane % CH;
+        u32x4 ov[NIT];
+        if (own_delta) {
+            const __bf16* obase = (const __bf16*)a.o.ptr + b * a.o.stride_b + h * a.o.stride_h + oc * 8;
+#pragma unroll
+            for (int it = 0; it < NIT; ++it)
+                ov[it] = *(const u32x4*)(obase + (int64_t)min(qw_lo + it * RPI + orow, a.S - 1) * a.o.stride_s);
+        }
         wait_vmem();
         __syncthreads();
 #pragma unroll
@@ -381,6 +396,35 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dq_bf16_kernel(AttnArgs 
             qf[kk] = TL::row_frag(Kbuf(0), rbase, 32 * w, kk);
             gf[kk] = TL::row_frag(Kbuf(1), rbase, 32 * w, kk);
         }
+        if (own_delta) {
+            // partial dot product per (row, chunk) -> per-wave LDS scratch [32 rows][CH] -> row sums
+            MA_LDS float* part = (MA_LDS float*)(lds0 + 4 * TL::bytes(BN) + 2 * BN * 8) + w * 32 * CH;
+#pragma unroll
+            for (int it = 0; it < NIT; ++it) {
+                const int row = it * RPI + orow;
+                const u32x4 g = *(MA_LDS u32x4*)(Kbuf(1) + TL::off(32 * w + row, oc * 8));
+                float acc = 0.f;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {  // bf16 -> fp32 is a 16-bit shift
+                    acc += __builtin_bit_cast(float, ov[it][e] << 16) * __builtin_bit_cast(float, g[e] << 16);
+                    acc += __builtin_bit_cast(float, ov[it][e] & 0xffff0000u) * __builtin_bit_cast(float, g[e] & 0xffff0000u);
+                }
+                part[row * CH + oc] = acc;
+            }
+            // lane (r, hh) sums half of row r's chunks; the other half comes from lane (r, 1 - hh)
+            float sum = 0.f;
+#pragma unroll
+            for (int c4 = 0; c4 < CH / 8; ++c4) {
+                const f32x4 p4 = *(MA_LDS f32x4*)(part + r * CH + hh * (CH / 2) + 4 * c4);
+                sum += (p4[0] + p4[1]) + (p4[2] + p4[3]);
+            }
+            delta = sum + xor32(sum);
+            if (qvalid && hh == 0) a.delta[rowi] = delta;
+        }
+        // From here on the fragments are MFMA operands only: move them to AGPRs once, now.  (Left to
+        // the register allocator, fragments that were also read by the vector ALU stay in VGPRs and
+        // get copied to AGPRs right in front of every MFMA that uses them.)
+        static_for<0, KK>([&](auto kk) { park_in_agprs(qf[decltype(kk)::value], gf[decltype(kk)::value]); });
         __syncthreads();
     }
 
@@ -550,9 +594,20 @@ static int bwd_dd(const AttnArgs& a, hipStream_t st) {
     constexpr int RPB = 256 / (D / 8);
     const int64_t nrows = (int64_t)a.B * a.Hq * a.S;
     int rc = MA_OK;
-    if (a.stages & MA_BWD_DELTA) {
+    // delta on its own only when the dQ stage, which computes it for its own rows, is not asked for
+    if ((a.stages & MA_BWD_DELTA) && !(a.stages & MA_BWD_DQ)) {
         hipLaunchKernelGGL(attn_delta_bf16_kernel<D>, dim3((unsigned)((nrows + RPB - 1) / RPB)), dim3(256), 0, st, a);
         rc = check_launch("attn_delta_bf16_kernel");
+        if (rc) return rc;
+    }
+    if (a.stages & MA_BWD_DQ) {  // first: the dK/dV kernel reads the delta this one may be writing
+        // K/V ring, kv document ids, and the per-wave scratch of the delta row sums
+        const size_t lds_q = (size_t)4 * Tile<D>::bytes(kStep) + 2 * kStep * 8 + (size_t)(kBwdThreads / 64) * 32 * (D / 8) * 4;
+        rc = opt_in_lds(attn_bwd_dq_bf16_kernel<D, HAS_DOC>, lds_q, "attn_bwd_dq_bf16");
+        if (rc) return rc;
+        hipLaunchKernelGGL((attn_bwd_dq_bf16_kernel<D, HAS_DOC>), dim3(work_grid(a.B * a.T, a.Hkv, a.Hq / a.Hkv), 1, 1), dim3(kBwdThreads),
+                           lds_q, st, a);
+        rc = check_launch("attn_bwd_dq_bf16_kernel");
         if (rc) return rc;
     }
     if (a.stages & MA_BWD_DKV) {
@@ -562,15 +617,8 @@ static int bwd_dd(const AttnArgs& a, hipStream_t st) {
         hipLaunchKernelGGL((attn_bwd_dkv_bf16_kernel<D, HAS_DOC>), dim3(work_grid(a.B * a.T, a.Hkv, 1), 1, 1), dim3(kBwdThreads), lds_kv,
                            st, a);
         rc = check_launch("attn_bwd_dkv_bf16_kernel");
-        if (rc) return rc;
     }
-    if (!(a.stages & MA_BWD_DQ)) return MA_OK;
-    const size_t lds_q = (size_t)4 * Tile<D>::bytes(kStep) + 2 * kStep * 8;
-    rc = opt_in_lds(attn_bwd_dq_bf16_kernel<D, HAS_DOC>, lds_q, "attn_bwd_dq_bf16");
-    if (rc) return rc;
-    hipLaunchKernelGGL((attn_bwd_dq_bf16_kernel<D, HAS_DOC>), dim3(work_grid(a.B * a.T, a.Hkv, a.Hq / a.Hkv), 1, 1), dim3(kBwdThreads),
-                       lds_q, st, a);
-    return check_launch("attn_bwd_dq_bf16_kernel");
+    return rc;
 }
 
 template <int D>

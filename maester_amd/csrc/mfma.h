@@ -26,6 +26,7 @@ namespace ma {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -125,6 +126,8 @@ __device__ __forceinline__ void mfma32_vv_zero(f32x16& c, bf16x8 a, bf16x8 b) {
 __device__ __forceinline__ void mfma32_acc_a(f32x16& c, bf16x8 a, bf16x8 b) {
     asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
 }
+// pins two operand fragments to AGPRs at this point of the program
+__device__ __forceinline__ void park_in_agprs(bf16x8& x, bf16x8& y) { asm volatile("" : "+a"(x), "+a"(y)); }
 // 16 wait states: enough for the result of an 8-pass MFMA to be readable by the vector ALU.  The
 // tiles are read-write operands so that nothing that uses them can be scheduled above the fence
 // (volatile asm statements keep their order among themselves).
