@@ -48,13 +48,12 @@ __device__ __forceinline__ void store8<float>(float* p, const float* v) {
 }
 template <>
 __device__ __forceinline__ void store8<uint16_t>(uint16_t* p, const float* v) {
-    uint4 a;
-    uint32_t w[4];
+    // the hardware conversion (v_cvt_pk_bf16_f32) rounds to nearest even like torch's cast
+    typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+    bf16x8_t o;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-        w[i] = (uint32_t)f32_to_bf16_bits(v[2 * i]) | ((uint32_t)f32_to_bf16_bits(v[2 * i + 1]) << 16);
-    a.x = w[0]; a.y = w[1]; a.z = w[2]; a.w = w[3];
-    *(uint4*)p = a;
+    for (int i = 0; i < 8; ++i) o[i] = (__bf16)v[i];
+    *(bf16x8_t*)p = o;
 }
 
 template <int LPH>
@@ -312,7 +311,21 @@ static int bwd_t(const ma_tensor4& qi, const ma_tensor4& ki, const ma_tensor4& d
                  const ma_tensor4& dqi, const ma_tensor4& dki, const float* qw, const float* kw, const float* cs,
                  const float* sn, const int64_t* pos, int64_t n_pos, int unit, const float* q_rstd,
                  const float* k_rstd, float* dqw, float* dkw, void* ws, int B, int S, int Hq, int Hkv, hipStream_t st) {
-    const int grid = prologue_bwd_blocks(B, S);
+    // One resident wave set: the kernel walks tokens with a grid stride, so a grid larger than what
+    // the device holds at once only adds a ragged second round (the workspace is sized for the cap).
+    int grid = prologue_bwd_blocks(B, S);
+    {
+        static int resident = 0;  // blocks of this instantiation the current device holds at once
+        if (resident == 0) {
+            int dev = 0, cus = 0, per_cu = 0;
+            if (hipGetDevice(&dev) == hipSuccess &&
+                hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess &&
+                hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, prologue_bwd_kernel<T, D>, 64 * kWavesPerBlock, 0) == hipSuccess)
+                resident = cus * per_cu;
+            if (resident <= 0) resident = 1024;
+        }
+        if (grid > resident) grid = resident;
+    }
     float* partials = (qw || kw) ? (float*)ws : nullptr;
     hipLaunchKernelGGL((prologue_bwd_kernel<T, D>), dim3(grid), dim3(64 * kWavesPerBlock), 0, st, qi, ki, dqo, dko,
                        dqi, dki, qw, kw, cs, sn, pos, n_pos, unit, q_rstd, k_rstd, partials, B, S, Hq, Hkv);
