@@ -90,7 +90,9 @@ const char* ma_last_error(void) { return g_err; }
 size_t ma_tile_map_workspace_bytes(int B, int S) {
     if (B <= 0 || S <= 0) return 0;
     const size_t T = ((size_t)S + MA_TILE - 1) / MA_TILE;
-    return (size_t)B * T * T;  // one class byte per tile
+    // class byte per tile (rounded up to 16 bytes) | (min, max) document id per tile | counter | list of
+    // the tiles that need an exact count
+    return (((size_t)B * T * T + 15) & ~(size_t)15) + (size_t)B * T * 2 * sizeof(int64_t) + 16 + (size_t)B * T * T * sizeof(int32_t);
 }
 
 int ma_tile_map_build(const int64_t* document_ids, int B, int S, int causal, int64_t window, const ma_tile_map* out,

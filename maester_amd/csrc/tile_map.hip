@@ -3,51 +3,111 @@
 // Stands in for create_block_mask(make_document_mask_wrapper(...), B, None, S, S)
 // (maester/models/gemma/model.py:694-730), which materialises a [B,1,S,S] bool and block-reduces
 // it (torch/nn/attention/flex_attention.py:979-1022, 429-441).  Here every 128x128 tile is
-// classified directly from the two 128-id slices it covers (exact for arbitrary ids, no S^2
-// memory), then the ordered lists are emitted: set tiles ascending, unset tiles ascending.
+// classified from the document ids of the two 128-row slices it covers (exact for arbitrary ids,
+// no S^2 memory): first by their (min, max) id ranges, and only the tiles the ranges cannot settle
+// by an exact 128x128 count; then the ordered lists are emitted: set tiles ascending, unset tiles
+// ascending.
 #include "common.h"
 
 namespace ma {
 
 // class codes in the workspace: 0 empty, 1 partial, 2 full
-__global__ __launch_bounds__(kTile) void classify_tiles_kernel(const int64_t* __restrict__ doc, int S, int T,
-                                                                int causal, int64_t window,
-                                                                uint8_t* __restrict__ cls) {
-    const int j = blockIdx.x, i = blockIdx.y, b = blockIdx.z;
-    uint8_t* out = cls + ((size_t)b * T + i) * T + j;
-    const int q0 = i * kTile, k0 = j * kTile;
-    // tiles the base predicate rules out entirely (uniform over the workgroup)
-    bool dead = false;
-    if ((causal || window >= 0) && k0 > q0 + kTile - 1) dead = true;
-    if (window >= 0 && (int64_t)q0 - (int64_t)(k0 + kTile - 1) > window) dead = true;
-    if (dead) {
-        if (threadIdx.x == 0) *out = 0;
-        return;
+
+// (min, max) document id over the valid rows of every 128-row tile; one wave per tile.  Also clears
+// the counter of the hard-tile list.  With doc == nullptr only the counter is cleared.
+__global__ __launch_bounds__(256) void tile_ranges_kernel(const int64_t* __restrict__ doc, int B, int S, int T,
+                                                          int64_t* __restrict__ rng, int* __restrict__ n_hard) {
+    if (blockIdx.x == 0 && threadIdx.x == 0) *n_hard = 0;
+    const int tile = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (!doc || tile >= B * T) return;
+    const int b = tile / T, r0 = (tile % T) * kTile;
+    const int64_t* row = doc + (size_t)b * S;
+    const int last = S - 1;
+    int64_t lo = row[min(r0 + lane, last)], hi = lo;
+    const int64_t x = row[min(r0 + 64 + lane, last)];
+    lo = min(lo, x);
+    hi = max(hi, x);
+    for (int off = 32; off > 0; off >>= 1) {
+        lo = min(lo, __shfl_xor(lo, off, 64));
+        hi = max(hi, __shfl_xor(hi, off, 64));
     }
+    if (lane == 0) {
+        rng[(size_t)tile * 2] = lo;
+        rng[(size_t)tile * 2 + 1] = hi;
+    }
+}
+
+// One thread per tile.  Most tiles are settled without looking at a single pair:
+//   * ruled out by the causal / window bound, or by disjoint document-id ranges      -> empty
+//   * both tiles hold one and the same document, every pair passes the bound, and the tile lies
+//     inside the sequence                                                              -> full
+// The rest (the diagonal, tiles a document boundary runs through, ragged edges) go on a list and are
+// counted exactly by count_hard_tiles_kernel.
+__global__ __launch_bounds__(256) void classify_easy_kernel(const int64_t* __restrict__ rng, int has_doc, int B, int S, int T,
+                                                             int causal, int64_t window, uint8_t* __restrict__ cls,
+                                                             int* __restrict__ n_hard, int32_t* __restrict__ hard) {
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (int64_t)B * T * T) return;
+    const int j = (int)(idx % T), i = (int)((idx / T) % T), b = (int)(idx / ((int64_t)T * T));
+    const int q0 = i * kTile, k0 = j * kTile;
+    const bool bounded = causal || window >= 0;
+    bool dead = bounded && k0 > q0 + kTile - 1;
+    if (window >= 0 && (int64_t)q0 - (int64_t)(k0 + kTile - 1) > window) dead = true;
+    int c = -1;  // undecided
+    if (dead) c = 0;
+    else if (has_doc) {
+        const int64_t* rrow = rng + (size_t)b * T * 2;
+        const int64_t qlo = rrow[2 * i], qhi = rrow[2 * i + 1], klo = rrow[2 * j], khi = rrow[2 * j + 1];
+        if (klo > qhi || khi < qlo) c = 0;
+        else if (klo == khi && qlo == qhi && klo == qlo) c = -2;  // one document on both sides
+    } else c = -2;                                                // no document term
+    if (c == -2) {
+        bool all = q0 + kTile <= S && k0 + kTile <= S;
+        if (bounded && !(q0 >= k0 + kTile - 1)) all = false;
+        if (window >= 0 && (int64_t)(q0 + kTile - 1) - (int64_t)k0 > window) all = false;
+        c = all ? 2 : -1;
+    }
+    if (c >= 0) cls[idx] = (uint8_t)c;
+    else hard[atomicAdd(n_hard, 1)] = (int32_t)idx;
+}
+
+// Exact class of the listed tiles: 128 x 128 compares from the two 128-id slices, as torch's dense
+// mask would give.  One workgroup per listed tile (grid-stride over the list).
+__global__ __launch_bounds__(kTile) void count_hard_tiles_kernel(const int64_t* __restrict__ doc, int S, int T, int causal,
+                                                                 int64_t window, uint8_t* __restrict__ cls,
+                                                                 const int* __restrict__ n_hard,
+                                                                 const int32_t* __restrict__ hard) {
     __shared__ int64_t kdoc[kTile];
     __shared__ int wave_cnt[kTile / 64];
     const int t = threadIdx.x;
-    const int64_t* drow = doc ? doc + (size_t)b * S : nullptr;
-    if (drow) kdoc[t] = (k0 + t < S) ? drow[k0 + t] : 0;
-    __syncthreads();
-    const int q = q0 + t;
-    int cnt = 0;
-    if (q < S) {
-        const int64_t dq = drow ? drow[q] : 0;
-        const int kmax = min(kTile, S - k0);
-        for (int c = 0; c < kmax; ++c) {
-            bool ok = pair_allowed(q, k0 + c, causal, window);
-            if (drow) ok = ok && (kdoc[c] == dq);
-            cnt += ok ? 1 : 0;
+    const int n = *n_hard;
+    for (int e = blockIdx.x; e < n; e += gridDim.x) {
+        const int64_t idx = hard[e];
+        const int j = (int)(idx % T), i = (int)((idx / T) % T), b = (int)(idx / ((int64_t)T * T));
+        const int q0 = i * kTile, k0 = j * kTile;
+        const int64_t* drow = doc ? doc + (size_t)b * S : nullptr;
+        if (drow) kdoc[t] = (k0 + t < S) ? drow[k0 + t] : 0;
+        __syncthreads();
+        const int q = q0 + t;
+        int cnt = 0;
+        if (q < S) {
+            const int64_t dq = drow ? drow[q] : 0;
+            const int kmax = min(kTile, S - k0);
+            for (int c = 0; c < kmax; ++c) {
+                bool ok = pair_allowed(q, k0 + c, causal, window);
+                if (drow) ok = ok && (kdoc[c] == dq);
+                cnt += ok ? 1 : 0;
+            }
         }
-    }
-    for (int off = 32; off > 0; off >>= 1) cnt += __shfl_down(cnt, off, 64);
-    if ((t & 63) == 0) wave_cnt[t >> 6] = cnt;
-    __syncthreads();
-    if (t == 0) {
-        int total = 0;
-        for (int w = 0; w < kTile / 64; ++w) total += wave_cnt[w];
-        *out = total == 0 ? 0 : (total == kTile * kTile ? 2 : 1);
+        for (int off = 32; off > 0; off >>= 1) cnt += __shfl_down(cnt, off, 64);
+        if ((t & 63) == 0) wave_cnt[t >> 6] = cnt;
+        __syncthreads();
+        if (t == 0) {
+            int total = 0;
+            for (int w = 0; w < kTile / 64; ++w) total += wave_cnt[w];
+            cls[idx] = total == 0 ? 0 : (total == kTile * kTile ? 2 : 1);
+        }
+        __syncthreads();
     }
 }
 
@@ -137,9 +197,22 @@ __global__ __launch_bounds__(256) void block_ranges_kernel(const int64_t* __rest
 int launch_tile_map(const int64_t* doc, int B, int S, int causal, int64_t window, const ma_tile_map& out,
                     void* ws, hipStream_t st) {
     const int T = (S + kTile - 1) / kTile;
+    // workspace: class bytes | tile id ranges | hard-tile counter | hard-tile list
     uint8_t* cls = (uint8_t*)ws;
-    hipLaunchKernelGGL(classify_tiles_kernel, dim3(T, T, B), dim3(kTile), 0, st, doc, S, T, causal, window, cls);
-    int rc = check_launch("classify_tiles_kernel");
+    const size_t ntiles = (size_t)B * T * T;
+    int64_t* rng = (int64_t*)((char*)ws + ((ntiles + 15) & ~(size_t)15));
+    int* n_hard = (int*)(rng + (size_t)B * T * 2);
+    int32_t* hard = (int32_t*)((char*)n_hard + 16);
+    hipLaunchKernelGGL(tile_ranges_kernel, dim3((B * T + 3) / 4), dim3(256), 0, st, doc, B, S, T, rng, n_hard);
+    int rc = check_launch("tile_ranges_kernel");
+    if (rc) return rc;
+    hipLaunchKernelGGL(classify_easy_kernel, dim3((unsigned)((ntiles + 255) / 256)), dim3(256), 0, st, rng, doc ? 1 : 0, B, S, T,
+                       causal, window, cls, n_hard, hard);
+    rc = check_launch("classify_easy_kernel");
+    if (rc) return rc;
+    hipLaunchKernelGGL(count_hard_tiles_kernel, dim3((unsigned)(ntiles < 4096 ? ntiles : 4096)), dim3(kTile), 0, st, doc, S, T,
+                       causal, window, cls, n_hard, hard);
+    rc = check_launch("count_hard_tiles_kernel");
     if (rc) return rc;
     hipLaunchKernelGGL(order_lists_kernel, dim3(T, B, 4), dim3(64), 0, st, cls, T, out);
     rc = check_launch("order_lists_kernel");

@@ -43,8 +43,9 @@ def _err():
 
 def test_workspace_sizes():
     L = _lib.lib()
-    assert L.ma_tile_map_workspace_bytes(4, 8192) == 4 * 64 * 64
-    assert L.ma_tile_map_workspace_bytes(1, 129) == 4
+    # class byte per tile + (min, max) int64 per tile row + counter + list of tiles to count exactly
+    assert L.ma_tile_map_workspace_bytes(4, 8192) == 4 * 64 * 64 + 4 * 64 * 16 + 16 + 4 * 64 * 64 * 4
+    assert L.ma_tile_map_workspace_bytes(1, 129) == 16 + 2 * 16 + 16 + 4 * 4   # T = 2: 4 class bytes rounded up to 16
     assert L.ma_tile_map_workspace_bytes(0, 10) == 0
     assert L.ma_attn_bwd_workspace_bytes(4, 8192, 8, 4, 256) == 4 * 8 * 8192 * 4
     assert L.ma_prologue_bwd_workspace_bytes(4, 8192, 8, 4, 256) > 0
