@@ -191,7 +191,7 @@ struct DocRange2 {     // two consecutive blocks (one 64-row step)
     __device__ __forceinline__ int64_t lo(int k) const { return (int64_t)(((uint64_t)(uint32_t)raw[4 * k + 1] << 32) | (uint32_t)raw[4 * k]); }
     __device__ __forceinline__ int64_t hi(int k) const { return (int64_t)(((uint64_t)(uint32_t)raw[4 * k + 3] << 32) | (uint32_t)raw[4 * k + 2]); }
     // can block k share a document with rows whose ids span [own_lo, own_hi]?
-    __device__ __forceinline__ bool meets(int k, int64_t own_lo, int64_t own_hi) const { return (lo(k) <= own_hi) & (hi(k) >= own_lo); }
+    __device__ __forceinline__ bool meets(int k, int64_t own_lo, int64_t own_hi) const { return (int)(lo(k) <= own_hi) & (int)(hi(k) >= own_lo); }
 };
 
 __device__ __forceinline__ int opaque_lane_zero() {

@@ -236,10 +236,12 @@ __device__ __forceinline__ void rowfrag_gemm(uint32_t row_addr, const bf16x8* re
     mfma_fence_tiles<NB>(acc);
 }
 
-// Two independent products of that kind at once, from two LDS tiles, interleaved MFMA by MFMA so
-// that consecutive MFMAs never depend on each other:
+// Two independent products of that kind, from two LDS tiles, in one read pipeline:
 //   acc0 = sum_kk L0(rows r, cols 16kk..) x reg0[kk],  acc1 = sum_kk L1(...) x reg1[kk].
-template <int D, int P, bool SWAP = false, bool REG_A = true, typename Hook = NoHook>
+// SEQ = false interleaves them MFMA by MFMA; SEQ = true finishes acc0 (MFMAs 0..KK-1) before acc1
+// (MFMAs KK..2KK-1), so that hooks of the second half can already work on acc0 with the vector ALU
+// (from MFMA KK+1 on: the result of an MFMA is readable two MFMAs later).
+template <int D, int P, bool SWAP = false, bool REG_A = true, typename Hook = NoHook, bool SEQ = false>
 __device__ __forceinline__ void rowfrag_gemm2(uint32_t row_addr0, const bf16x8* reg0, f32x16& acc0, uint32_t row_addr1,
                                               const bf16x8* reg1, f32x16& acc1, Hook&& hook = Hook{}) {
     constexpr int KK = D / 16;
@@ -247,25 +249,29 @@ __device__ __forceinline__ void rowfrag_gemm2(uint32_t row_addr0, const bf16x8* 
     bf16x8 t[N];
     auto rd = [&](auto idx) {
         constexpr int i = decltype(idx)::value;
-        constexpr int kk = i / 2, which = i % 2;
+        constexpr int kk = SEQ ? i % KK : i / 2, which = SEQ ? i / KK : i % 2;
         t[i] = lds_read_b128<kk * 32>(which ? row_addr1 : row_addr0);
     };
     auto step = [&](auto idx) {
         constexpr int i = decltype(idx)::value;
-        constexpr int kk = i / 2, which = i % 2;
+        constexpr int kk = SEQ ? i % KK : i / 2, which = SEQ ? i / KK : i % 2;
         constexpr int younger = (N - 1 - i) < (P - 1) ? (N - 1 - i) : (P - 1);
         lds_wait<younger>(t[i]);
-        f32x16& acc = which ? acc1 : acc0;
-        const bf16x8 rg = which ? reg1[kk] : reg0[kk];
-        if constexpr (kk == 0) {
-            if constexpr (!REG_A) { if constexpr (SWAP) mfma32_vv_zero(acc, rg, t[i]); else mfma32_vv_zero(acc, t[i], rg); }
-            else if constexpr (SWAP) mfma32_av_zero(acc, rg, t[i]);
-            else mfma32_va_zero(acc, t[i], rg);
-        } else {
-            if constexpr (!REG_A) { if constexpr (SWAP) mfma32_vv(acc, rg, t[i]); else mfma32_vv(acc, t[i], rg); }
-            else if constexpr (SWAP) mfma32_av(acc, rg, t[i]);
-            else mfma32_va(acc, t[i], rg);
-        }
+        // the register fragment is handed to the asm statement as it is (no copy: a copy of an
+        // AGPR-resident fragment would need AGPRs of its own)
+        auto one = [&](f32x16& acc, const bf16x8& rg) {
+            if constexpr (kk == 0) {
+                if constexpr (!REG_A) { if constexpr (SWAP) mfma32_vv_zero(acc, rg, t[i]); else mfma32_vv_zero(acc, t[i], rg); }
+                else if constexpr (SWAP) mfma32_av_zero(acc, rg, t[i]);
+                else mfma32_va_zero(acc, t[i], rg);
+            } else {
+                if constexpr (!REG_A) { if constexpr (SWAP) mfma32_vv(acc, rg, t[i]); else mfma32_vv(acc, t[i], rg); }
+                else if constexpr (SWAP) mfma32_av(acc, rg, t[i]);
+                else mfma32_va(acc, t[i], rg);
+            }
+        };
+        if constexpr (which) one(acc1, reg1[kk]);
+        else one(acc0, reg0[kk]);
     };
     static_for<0, (P < N ? P : N)>(rd);
     static_for<0, N>([&](auto idx) {
@@ -283,15 +289,18 @@ __device__ __forceinline__ void rowfrag_gemm2(uint32_t row_addr0, const bf16x8* 
 // transposed fragments (tr_addr = lds address of the tile + Tile::tr_base(lane)).  Pipeline of
 // depth P over the NJ * DB fragments (two LDS reads each).  reg lives in VGPRs, acc in VGPRs or
 // (ACC_A) AGPRs; ends with mfma_fence().
-template <int D, int NJ, int P, bool ACC_A = false, typename Hook = NoHook>
+// READY: how many of the reg fragments are complete when the chain starts; the others are
+// produced by the hooks of earlier MFMAs (fragment j is first used by MFMA j*DB) and are picked up
+// from reg_in just before their first use.
+template <int D, int NJ, int P, bool ACC_A = false, typename Hook = NoHook, int READY = NJ>
 __device__ __forceinline__ void trfrag_gemm(uint32_t tr_addr, const bf16x8* reg_in, f32x16* acc, Hook&& hook = Hook{}) {
     using TL = Tile<D>;
     constexpr int DB = D / 32;
     constexpr int N = NJ * DB;
     bf16x8 reg[NJ];
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) reg[j] = reg_in[j];
-    pin_frags<0, NJ>(reg);
+    for (int j = 0; j < READY; ++j) reg[j] = reg_in[j];
+    pin_frags<0, READY>(reg);
     bf16x4 lo[N], hi[N];
     auto rd = [&](auto idx) {
         constexpr int i = decltype(idx)::value;
@@ -303,6 +312,10 @@ __device__ __forceinline__ void trfrag_gemm(uint32_t tr_addr, const bf16x8* reg_
         constexpr int i = decltype(idx)::value;
         constexpr int j = i / DB, db = i % DB;
         constexpr int younger = (N - 1 - i) < (P - 1) ? (N - 1 - i) : (P - 1);
+        if constexpr (j >= READY && db == 0) {  // a fragment the hooks have just finished
+            reg[j] = reg_in[j];
+            asm volatile("s_nop 4" : "+v"(reg[j]));
+        }
         // wait on the two halves themselves: a copy made while assembling the 8-element fragment
         // must not read them before the data has landed
         lds_wait2<2 * younger>(lo[i], hi[i]);
