@@ -179,7 +179,7 @@ __global__ __launch_bounds__(kFwdThreads) void attn_fwd_bf16_kernel(AttnArgs a) 
         // is masked below, and keeping one straight-line path keeps every accumulator in place.
         f32x16 s[2];
         rowfrag_gemm<D, 2, kPipe>(lds_addr(Ks) + rbase, qf, s, pace_k);
-        // scale into log2 units and mask
+        // mask (the scale into log2 units is folded into the exponent below)
         float mx = -INFINITY;
         if (cpartial) {
             // d = q - kv for element v is qrel - (32*nb + 8*(v/4) + v%4).  The causal, window and
@@ -209,7 +209,7 @@ __global__ __launch_bounds__(kFwdThreads) void attn_fwd_bf16_kernel(AttnArgs a) 
                         const int v = 4 * g + e;
                         bool ok = (t0 - (unsigned)(32 * nb + 8 * g + e) <= span) & some & act[nb];
                         if (HAS_DOC) ok = ok & (ids[g][e >> 1][e & 1] == docq);
-                        const float x = ok ? s[nb][v] * sl2 : -INFINITY;
+                        const float x = ok ? s[nb][v] : -INFINITY;
                         s[nb][v] = x;
                         mx = fmaxf(mx, x);
                     }
@@ -220,14 +220,11 @@ __global__ __launch_bounds__(kFwdThreads) void attn_fwd_bf16_kernel(AttnArgs a) 
 #pragma unroll
             for (int nb = 0; nb < 2; ++nb) {
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const float x = s[nb][v] * sl2;
-                    s[nb][v] = x;
-                    mx = fmaxf(mx, x);
-                }
+                for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[nb][v]);
             }
         }
-        mx = fmaxf(mx, xor32(mx));
+        // the scores stay unscaled: the (positive) scale goes into the exponent's multiply-add below
+        mx = fmaxf(mx, xor32(mx)) * sl2;
         // Lazy rescaling: the running reference m only moves when the row maximum has grown by more
         // than kSlack (in log2 units), so exp2(x - m) stays below 2^kSlack and the accumulator
         // rescale is a rare, wave-uniform branch instead of 128 multiplies per step.
@@ -250,7 +247,7 @@ __global__ __launch_bounds__(kFwdThreads) void attn_fwd_bf16_kernel(AttnArgs a) 
         for (int nb = 0; nb < 2; ++nb) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                const float p = fast_exp2(s[nb][v] - mu);
+                const float p = fast_exp2(__builtin_fmaf(s[nb][v], sl2, -mu));
                 rs += p;
                 pf[nb][v >> 3][v & 7] = (__bf16)p;
             }
