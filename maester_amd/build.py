@@ -16,7 +16,8 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(HERE, "csrc", "build")
 LIB_PATH = os.path.join(HERE, "libmaester_attn.so")
 
-SOURCES = ["api.hip", "tile_map.hip", "prologue.hip", "attn_f32.hip", "attn_fwd_bf16.hip", "attn_bwd_bf16.hip"]
+SOURCES = ["api.hip", "tile_map.hip", "prologue.hip", "attn_f32.hip", "attn_fwd_bf16.hip", "attn_fwd_pair_bf16.hip",
+           "attn_bwd_bf16.hip"]
 
 # -packed-fp32-ops is switched off on purpose: fp32 arithmetic is issued as scalar-per-lane VALU
 # instructions only.
@@ -48,7 +49,7 @@ def _compile(src: str, verbose: bool) -> str:
     return obj
 
 
-def build(verbose: bool = False, jobs: int = 6) -> str:
+def build(verbose: bool = False, jobs: int = 7) -> str:
     os.makedirs(OBJ_DIR, exist_ok=True)
     with ThreadPoolExecutor(max_workers=jobs) as ex:
         objs = list(ex.map(lambda s: _compile(s, verbose), SOURCES))

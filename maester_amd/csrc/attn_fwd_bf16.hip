@@ -310,6 +310,8 @@ static int fwd_d(const AttnArgs& a, hipStream_t st) {
 }
 
 int launch_attn_fwd_bf16(const AttnArgs& a, hipStream_t st) {
+    // query heads that share a kv head are processed in pairs when they come in pairs
+    if ((a.Hq / a.Hkv) % 2 == 0) return launch_attn_fwd_pair_bf16(a, st);
     switch (a.D) {
         case 64: return fwd_d<64>(a, st);
         case 128: return fwd_d<128>(a, st);

@@ -1,0 +1,339 @@
+// GQA flash-style forward for bf16 activations, two query heads per workgroup.
+//
+// Same contract as attn_fwd_bf16_kernel (maester/models/gemma/model.py:384-396; semantics
+// torch/_higher_order_ops/flex_attention.py:159-267), for head layouts where an even number of
+// query heads shares each kv head (enable_gqa, model.py:395).  A workgroup owns a 128-row q tile of
+// TWO query heads of one kv head; wave w owns rows 32w..32w+31 of both.  The two heads read the
+// same K and V, have the same mask and walk the same kv list, so per kv step the workgroup
+//   * stages K/V once (half the global -> LDS traffic per FLOP),
+//   * reads every K row fragment and every transposed V fragment from LDS once and feeds it to two
+//     MFMAs (half the LDS reads per MFMA: the transposed reads bound the single-head kernel),
+//   * evaluates the mask once,
+// and the per-step control, the barrier and the per-workgroup prologue/epilogue are paid once for
+// twice the work.  The price is registers: both O^T accumulators fill all 256 AGPRs, both heads' Q
+// fragments take 128 VGPRs, so the 64-row kv step is consumed as two 32-row blocks.
+//
+// With the accumulators in AGPRs and no register to spare, there is no cheap way to multiply O^T by
+// a per-row factor, so the online softmax never rescales: a row's reference maximum is set by its
+// first visible block and exp2(score - reference) may grow up to 2^kSlack (exact in fp32 / bf16, a
+// power-of-two scale).  If some row ever outgrows that, the workgroup notes it, finishes the walk,
+// and redoes its tile in two passes: one that only finds the exact row maxima, one that accumulates
+// against them.  That costs the workgroup half a forward more, and takes scores that span more than
+// kSlack * ln 2 (44 nats) above a row's first block to happen.
+#include "common.h"
+#include "mfma.h"
+
+namespace ma {
+
+constexpr int kPairThreads = 256;
+constexpr int kPairBN = 64;   // kv rows staged per step
+constexpr int kPairPipeK = 3;
+constexpr int kPairPipeV = 3;
+
+template <int D, bool HAS_DOC>
+__global__ __launch_bounds__(kPairThreads) void attn_fwd_pair_bf16_kernel(AttnArgs a) {
+    using TL = Tile<D>;
+    constexpr int KK = D / 16;
+    constexpr int DB = D / 32;
+    constexpr int BN = kPairBN;
+    constexpr int NW = kPairThreads / 64;
+    extern __shared__ __align__(16) char smem_raw[];
+    const lds_ptr lds0 = (lds_ptr)smem_raw;
+    auto Kbuf = [&](int i) { return lds0 + i * 2 * TL::bytes(BN); };
+    auto Vbuf = [&](int i) { return lds0 + i * 2 * TL::bytes(BN) + TL::bytes(BN); };
+    auto Dbuf = [&](int i) { return (MA_LDS int64_t*)(lds0 + 4 * TL::bytes(BN)) + i * BN; };
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 31, hh = lane >> 5;
+    const int G = a.Hq / a.Hkv, GP = G / 2;  // head pairs per kv head
+    int i, hp, b;
+    if (!map_work(blockIdx.x, a.B * a.T, a.T, a.Hkv, GP, a.map.q_tile_order, i, hp, b)) return;
+    const int hk = hp / GP;
+    const int h0 = hk * G + 2 * (hp % GP);   // the pair is (h0, h0 + 1)
+    const int qw_lo = i * kTile + 32 * w, qw_hi = qw_lo + 31;
+    const int q = qw_lo + r;
+    const bool qvalid = q < a.S;
+    const bool bounded = a.causal || a.window >= 0;
+
+    const __bf16* qp = (const __bf16*)a.q.ptr + b * a.q.stride_b + h0 * a.q.stride_h;
+    const char* kp = (const char*)((const __bf16*)a.k.ptr + b * a.k.stride_b + hk * a.k.stride_h);
+    const char* vp = (const char*)((const __bf16*)a.v.ptr + b * a.v.stride_b + hk * a.v.stride_h);
+    const uint32_t ksb = (uint32_t)(a.k.stride_s * 2), vsb = (uint32_t)(a.v.stride_s * 2);
+    const int64_t* drow = HAS_DOC ? a.doc + (size_t)b * a.S : nullptr;
+    const int rbase = TL::row_base(lane), tbase = TL::tr_base(lane);
+
+    // Both heads' Q tiles come in through LDS (coalesced), one per K/V buffer pair, and stay in VGPRs.
+    bf16x8 qa[KK], qb[KK];
+    {
+        DirectStager<D, kTile, NW> sq;
+        sq.init(w, lane);
+        const int rows_valid = min(kTile, a.S - i * kTile);
+        sq.issue(qp + (int64_t)i * kTile * a.q.stride_s, Kbuf(0), w, lane, rows_valid, a.q.stride_s);
+        sq.issue(qp + a.q.stride_h + (int64_t)i * kTile * a.q.stride_s, Kbuf(1), w, lane, rows_valid, a.q.stride_s);
+    }
+
+    const int qc = min(q, a.S - 1);
+    const int64_t docq = HAS_DOC ? drow[qc] : 0;
+    const bool windowed = a.window >= 0;
+    const int wlim = windowed ? (int)min(a.window, (int64_t)0x3fffffff) : 0x7fffffff;
+    const float sl2 = a.scale * kLog2e;
+
+    const size_t mrow = (size_t)b * a.T + i;
+    StepWalk<BN> st;
+    int blk_lo, blk_hi;
+    visibility_limits(false, qw_lo, qw_hi, 32, bounded, wlim, windowed, blk_lo, blk_hi);
+    const bool use_rng = HAS_DOC && a.map.block_doc_range != nullptr;
+    const int64_t* rng_row = use_rng ? a.map.block_doc_range + (size_t)b * (2 * ((a.S + 63) / 64)) * 2 : nullptr;
+    DocRange own;
+    if (use_rng) {
+        own.load(rng_row + (size_t)(min(qw_lo, a.S - 1) / MA_DOC_BLOCK) * 2);
+        own.ready();
+    }
+
+    DirectStager<D, BN, NW> sk;
+    sk.init(w, lane);
+    const int my_runs = decltype(sk)::runs_of(w);
+    int64_t kd_next = 0;
+
+    wait_vmem();
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+        qa[kk] = TL::row_frag(Kbuf(0), rbase, 32 * w, kk);
+        qb[kk] = TL::row_frag(Kbuf(1), rbase, 32 * w, kk);
+    }
+    __syncthreads();  // all Q fragments are in registers before the buffers are reused
+
+    // O^T of both heads: all 256 AGPRs (D = 256); nothing but MFMAs touches them inside the loop
+    f32x16 oa[DB], ob[DB];
+    float ma_ = -INFINITY, mb_ = -INFINITY, la = 0.f, lb = 0.f;
+    MA_LDS int* outgrown = (MA_LDS int*)(lds0 + 4 * TL::bytes(BN) + 2 * BN * 8);
+    if (tid == 0) *outgrown = 0;
+    constexpr float kSlack = 32.0f;
+
+    // mode 0: the one pass described above; mode 1: row maxima only; mode 2: accumulate against them
+    for (int mode = 0;; ) {
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) oa[db][v] = ob[db][v] = 0.f;
+    pin_tiles<0, DB, true>(oa);
+    pin_tiles<0, DB, true>(ob);
+    la = lb = 0.f;
+    if (mode != 2) ma_ = mb_ = -INFINITY;
+    {
+        int lo, hi;
+        visibility_limits(false, i * kTile, i * kTile + kTile - 1, BN, bounded, wlim, windowed, lo, hi);
+        st.init(a.map.kv_indices + mrow * a.T, a.map.kv_num_blocks[mrow], a.map.full_kv_indices + mrow * a.T,
+                a.map.full_kv_num_blocks[mrow], 1, false, a.S, lo, hi);
+    }
+    bool have = st.next();
+    int k0 = st.r0;
+    bool partial = st.partial;
+    if (have) {
+        const int rows_valid = min(BN, a.S - k0);
+        sk.issue((const __bf16*)(kp + (uint64_t)(uint32_t)k0 * ksb), Kbuf(0), w, lane, rows_valid, a.k.stride_s);
+        sk.issue((const __bf16*)(vp + (uint64_t)(uint32_t)k0 * vsb), Vbuf(0), w, lane, rows_valid, a.v.stride_s);
+        if (HAS_DOC && partial && tid < BN) kd_next = drow[min(k0 + tid, a.S - 1)];
+    }
+
+    for (int n = 0; have; ++n) {
+        const int cur = n & 1;
+        const lds_ptr Ks = Kbuf(cur), Vs = Vbuf(cur);
+        MA_LDS int64_t* kdoc = Dbuf(cur);
+        DocRange2 rng;
+        if (use_rng && partial) rng.load(rng_row + (size_t)(k0 / MA_DOC_BLOCK) * 2);
+        if (HAS_DOC && partial && tid < BN) kdoc[tid] = kd_next;
+        wait_vmem();
+        __syncthreads();
+
+        const int ck0 = k0;
+        const bool cpartial = partial;
+        have = st.next();
+        bool act[2];
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) act[nb] = block_visible(ck0 + 32 * nb, a.S, cpartial, blk_lo, blk_hi);
+        if (use_rng && cpartial) {
+            rng.ready();
+#pragma unroll
+            for (int nb = 0; nb < 2; ++nb) act[nb] &= rng.meets(nb, own.lo(), own.hi());
+        }
+        // the tile loads of the next step ride in the chains of the first active block (K in its S^T
+        // chain, V in its O^T chain); a ragged last tile or a step without chains issues them at once
+        int pace = 0;
+        const char *ksrc = kp, *vsrc = vp;
+        const int first = act[0] ? 0 : 1;
+        if (have) {
+            k0 = st.r0;
+            partial = st.partial;
+            ksrc = kp + (uint64_t)(uint32_t)k0 * ksb;
+            vsrc = vp + (uint64_t)(uint32_t)k0 * vsb;
+            if (HAS_DOC && partial && tid < BN) kd_next = drow[min(k0 + tid, a.S - 1)];
+            pace = __builtin_amdgcn_readfirstlane(((k0 + BN <= a.S) & (act[0] | act[1]) & (mode != 1)) ? my_runs : 0);
+            if (!pace) {
+                const int rows_valid = min(BN, a.S - k0);
+                sk.issue((const __bf16*)ksrc, Kbuf(cur ^ 1), w, lane, rows_valid, a.k.stride_s);
+                sk.issue((const __bf16*)vsrc, Vbuf(cur ^ 1), w, lane, rows_valid, a.v.stride_s);
+            }
+        }
+        const uint32_t kdst = lds_addr(Kbuf(cur ^ 1)), vdst = lds_addr(Vbuf(cur ^ 1));
+
+        // mask constants of this step (see attn_fwd_bf16_kernel)
+        const int qrel = q - ck0 - 4 * hh;
+        const int dlo = max(bounded ? 0 : -0x40000000, q - a.S + 1);
+        const unsigned span = (unsigned)(wlim - dlo);
+        const bool some = wlim >= dlo;
+        const unsigned t0 = (unsigned)(qrel - dlo);
+
+#pragma unroll 1
+        for (int nb = 0; nb < 2; ++nb) {
+            if (!(nb ? act[1] : act[0])) continue;
+            const int lim = nb == first ? pace : 0;
+            constexpr int kEvery = (2 * KK) / decltype(sk)::PER;  // both chains have 2*KK MFMAs
+            static_assert(kEvery >= 1 && 4 * DB == 2 * KK, "pacing");
+            auto pace_k = [&](auto idx) {
+                constexpr int c = decltype(idx)::value;
+                if constexpr (c % kEvery == kEvery - 1) sk.template issue_one<c / kEvery>((const __bf16*)ksrc, kdst, w, lim, ksb);
+            };
+            auto pace_v = [&](auto idx) {
+                constexpr int c = decltype(idx)::value;
+                if constexpr (c % kEvery == kEvery - 1) sk.template issue_one<c / kEvery>((const __bf16*)vsrc, vdst, w, lim, vsb);
+            };
+            const uint32_t roff = (uint32_t)(32 * nb * TL::kPitch);
+
+            // S^T of both heads for 32 kv rows (lane owns one q row, 16 of the kv rows)
+            f32x16 sa, sb;
+            rowfrag_gemm_dual<D, kPairPipeK>(lds_addr(Ks) + rbase + roff, qa, qb, sa, sb, pace_k);
+
+            // mask (shared by the two heads) and row maxima on the unscaled scores
+            float mxa = -INFINITY, mxb = -INFINITY;
+            if (cpartial) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    i64x2 id01 = {0, 0}, id23 = {0, 0};
+                    if (HAS_DOC) {
+                        id01 = *(MA_LDS i64x2*)(kdoc + 32 * nb + 8 * g + 4 * hh);
+                        id23 = *(MA_LDS i64x2*)(kdoc + 32 * nb + 8 * g + 4 * hh + 2);
+                    }
+                    const int64_t ids[4] = {id01[0], id01[1], id23[0], id23[1]};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int v = 4 * g + e;
+                        bool ok = (t0 - (unsigned)(32 * nb + 8 * g + e) <= span) & some;
+                        if (HAS_DOC) ok = ok & (ids[e] == docq);
+                        sa[v] = ok ? sa[v] : -INFINITY;
+                        sb[v] = ok ? sb[v] : -INFINITY;
+                        mxa = fmaxf(mxa, sa[v]);
+                        mxb = fmaxf(mxb, sb[v]);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    mxa = fmaxf(mxa, sa[v]);
+                    mxb = fmaxf(mxb, sb[v]);
+                }
+            }
+            mxa = fmaxf(mxa, xor32(mxa)) * sl2;   // the (positive) scale goes into the exponent's multiply-add
+            mxb = fmaxf(mxb, xor32(mxb)) * sl2;
+            if (mode == 1) {  // maxima only
+                ma_ = fmaxf(ma_, mxa);
+                mb_ = fmaxf(mb_, mxb);
+                continue;
+            }
+            if (mode == 0) {
+                // the first visible block sets the reference; a later block that outgrows it by more
+                // than kSlack log2 units sends the workgroup into the two-pass redo
+                const bool late = ((ma_ != -INFINITY) & (mxa > ma_ + kSlack)) | ((mb_ != -INFINITY) & (mxb > mb_ + kSlack));
+                if (__any(late) && lane == 0) *outgrown = 1;
+                ma_ = ma_ == -INFINITY ? mxa : ma_;
+                mb_ = mb_ == -INFINITY ? mxb : mb_;
+            }
+            const float mua = ma_ == -INFINITY ? 0.f : ma_, mub = mb_ == -INFINITY ? 0.f : mb_;
+            float rsa = 0.f, rsb = 0.f;
+            bf16x8 pa[2], pb[2];
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const float x = fast_exp2(__builtin_fmaf(sa[v], sl2, -mua));
+                const float y = fast_exp2(__builtin_fmaf(sb[v], sl2, -mub));
+                rsa += x;
+                rsb += y;
+                pa[v >> 3][v & 7] = (__bf16)x;
+                pb[v >> 3][v & 7] = (__bf16)y;
+            }
+            la += rsa + xor32(rsa);
+            lb += rsb + xor32(rsb);
+
+            // O^T += V^T P^T for both heads: every transposed V fragment feeds two MFMAs
+            trfrag_gemm_dual<D, 2, kPairPipeV>(lds_addr(Vs) + tbase + roff, pa, pb, oa, ob, pace_v);
+        }
+    }
+
+    __syncthreads();  // every wave is done with the K/V buffers, and with the flag
+    const int redo = *outgrown;
+    if (mode == 0 && redo) { mode = 1; continue; }
+    if (mode == 1) { mode = 2; continue; }
+    break;
+    }  // passes
+
+    // Epilogue: O^T (a lane owns one q row, 4 consecutive d per register group) goes through the
+    // wave's LDS scratch so that the global stores are whole 16-byte-per-lane row segments.
+    __syncthreads();  // every wave is done with the K/V buffers
+    mfma_fence();
+    {
+        constexpr int kPitchO = D * 2 + 16;
+        lds_ptr Os = lds0 + w * 32 * kPitchO;
+        constexpr int CH = D / 8, RPI = 64 / CH;
+        const int rsub = lane / CH, c = lane % CH;
+#pragma unroll 1
+        for (int hsel = 0; hsel < 2; ++hsel) {
+            const float l = hsel ? lb : la, m = hsel ? mb_ : ma_;
+            const float inv = l > 0.f ? 1.0f / l : 0.f;
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    bf16x4 pk;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) pk[e] = (__bf16)((hsel ? ob[db][4 * g + e] : oa[db][4 * g + e]) * inv);
+                    *(MA_LDS bf16x4*)(Os + r * kPitchO + (32 * db + 8 * g + 4 * hh) * 2) = pk;
+                }
+            }
+            __bf16* og = (__bf16*)a.o.ptr + b * a.o.stride_b + (h0 + hsel) * a.o.stride_h;
+#pragma unroll
+            for (int it = 0; it < 32 / RPI; ++it) {
+                const int row = it * RPI + rsub;
+                const u32x4 val = *(MA_LDS u32x4*)(Os + row * kPitchO + c * 16);
+                if (qw_lo + row < a.S) *(u32x4*)(og + (int64_t)(qw_lo + row) * a.o.stride_s + c * 8) = val;
+            }
+            if (qvalid && hh == 0)
+                a.lse[((size_t)b * a.Hq + h0 + hsel) * a.S + q] = l > 0.f ? (m + __log2f(l)) * kLn2 : -INFINITY;
+        }
+    }
+}
+
+template <int D, bool HAS_DOC>
+static int pair_dd(const AttnArgs& a, hipStream_t st) {
+    const size_t lds = (size_t)4 * Tile<D>::bytes(kPairBN) + 2 * kPairBN * 8 + 16;  // K/V ring, kv ids, redo flag
+    if (lds > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_pair_bf16_kernel<D, HAS_DOC>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return fail(MA_ERR_LAUNCH, "hipFuncSetAttribute(attn_fwd_pair_bf16, %zu): %s", lds, hipGetErrorString(e));
+    }
+    const int GP = a.Hq / a.Hkv / 2;
+    hipLaunchKernelGGL((attn_fwd_pair_bf16_kernel<D, HAS_DOC>), dim3(work_grid(a.B * a.T, a.Hkv, GP), 1, 1), dim3(kPairThreads), lds, st, a);
+    return check_launch("attn_fwd_pair_bf16_kernel");
+}
+
+// Only for head layouts with an even number of query heads per kv head; the caller checks.
+int launch_attn_fwd_pair_bf16(const AttnArgs& a, hipStream_t st) {
+    switch (a.D) {
+        case 64: return a.doc ? pair_dd<64, true>(a, st) : pair_dd<64, false>(a, st);
+        case 128: return a.doc ? pair_dd<128, true>(a, st) : pair_dd<128, false>(a, st);
+        case 256: return a.doc ? pair_dd<256, true>(a, st) : pair_dd<256, false>(a, st);
+    }
+    return fail(MA_ERR_UNSUPPORTED, "attn_fwd bf16: head_dim %d not in {64,128,256}", a.D);
+}
+
+}  // namespace ma

@@ -59,6 +59,7 @@ struct AttnArgs {
 int launch_attn_fwd_f32(const AttnArgs& a, hipStream_t st);
 int launch_attn_bwd_f32(const AttnArgs& a, hipStream_t st);
 int launch_attn_fwd_bf16(const AttnArgs& a, hipStream_t st);
+int launch_attn_fwd_pair_bf16(const AttnArgs& a, hipStream_t st);  // even number of q heads per kv head
 int launch_attn_bwd_bf16(const AttnArgs& a, hipStream_t st);
 
 // Workgroup id -> work item.  A unit is a tile row (q tile for the forward and dQ kernels, kv tile

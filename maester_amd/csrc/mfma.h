@@ -333,6 +333,77 @@ __device__ __forceinline__ void trfrag_gemm(uint32_t tr_addr, const bf16x8* reg_
     mfma_fence_tiles<DB, ACC_A>(acc);  // whatever comes next may read acc with the vector ALU
 }
 
+// ---- register-blocked variants: every LDS fragment feeds two MFMAs ---------------------------------
+// For two query heads that share a kv head, the K (or V) fragment read from LDS is the same for both:
+// reading it once halves the LDS traffic per MFMA (the transposed reads of the second product are
+// what bounds a single-head chain).  Hooks are numbered by MFMA (two per fragment).
+//
+// accA = sum_kk L(rows r, cols 16kk..) x regA[kk], accB = the same with regB; 32 rows of the tile at
+// row_addr; register fragments in VGPRs; accumulators (overwritten) in VGPRs.
+template <int D, int P, typename Hook = NoHook>
+__device__ __forceinline__ void rowfrag_gemm_dual(uint32_t row_addr, const bf16x8* regA, const bf16x8* regB, f32x16& accA,
+                                                  f32x16& accB, Hook&& hook = Hook{}) {
+    constexpr int N = D / 16;
+    bf16x8 t[N];
+    auto rd = [&](auto idx) {
+        constexpr int i = decltype(idx)::value;
+        t[i] = lds_read_b128<i * 32>(row_addr);
+    };
+    static_for<0, (P < N ? P : N)>(rd);
+    static_for<0, N>([&](auto idx) {
+        constexpr int i = decltype(idx)::value;
+        constexpr int younger = (N - 1 - i) < (P - 1) ? (N - 1 - i) : (P - 1);
+        lds_wait<younger>(t[i]);
+        if constexpr (i == 0) mfma32_vv_zero(accA, t[i], regA[i]);
+        else mfma32_vv(accA, t[i], regA[i]);
+        hook(std::integral_constant<int, 2 * i>{});
+        if constexpr (i == 0) mfma32_vv_zero(accB, t[i], regB[i]);
+        else mfma32_vv(accB, t[i], regB[i]);
+        if constexpr (i + P < N) rd(std::integral_constant<int, i + P>{});
+        hook(std::integral_constant<int, 2 * i + 1>{});
+    });
+    mfma_fence();
+    asm volatile("" : "+v"(accA));
+    asm volatile("" : "+v"(accB));
+}
+
+// accA[db] += L^T(rows 16j.., cols 32db..) x regA[j], accB[db] += the same x regB[j], over NJ
+// 16-row slabs of the tile at tr_addr; accumulators in AGPRs.
+template <int D, int NJ, int P, typename Hook = NoHook>
+__device__ __forceinline__ void trfrag_gemm_dual(uint32_t tr_addr, const bf16x8* regA_in, const bf16x8* regB_in, f32x16* accA,
+                                                 f32x16* accB, Hook&& hook = Hook{}) {
+    using TL = Tile<D>;
+    constexpr int DB = D / 32;
+    constexpr int N = NJ * DB;
+    bf16x8 regA[NJ], regB[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) { regA[j] = regA_in[j]; regB[j] = regB_in[j]; }
+    pin_frags<0, NJ>(regA);
+    pin_frags<0, NJ>(regB);
+    bf16x4 lo[N], hi[N];
+    auto rd = [&](auto idx) {
+        constexpr int i = decltype(idx)::value;
+        constexpr int j = i / DB, db = i % DB;
+        lo[i] = lds_read_tr16_b64<(16 * j) * TL::kPitch + db * 64>(tr_addr);
+        hi[i] = lds_read_tr16_b64<(16 * j + 2) * TL::kPitch + db * 64>(tr_addr);
+    };
+    static_for<0, (P < N ? P : N)>(rd);
+    static_for<0, N>([&](auto idx) {
+        constexpr int i = decltype(idx)::value;
+        constexpr int j = i / DB, db = i % DB;
+        constexpr int younger = (N - 1 - i) < (P - 1) ? (N - 1 - i) : (P - 1);
+        lds_wait2<2 * younger>(lo[i], hi[i]);
+        const bf16x8 f = __builtin_shufflevector(lo[i], hi[i], 0, 1, 2, 3, 4, 5, 6, 7);
+        mfma32_acc_a(accA[db], f, regA[j]);
+        hook(std::integral_constant<int, 2 * i>{});
+        mfma32_acc_a(accB[db], f, regB[j]);
+        if constexpr (i + P < N) rd(std::integral_constant<int, i + P>{});
+        hook(std::integral_constant<int, 2 * i + 1>{});
+    });
+    mfma_fence_tiles<DB, true>(accA);
+    pin_tiles<0, DB, true>(accB);
+}
+
 // Global -> registers -> LDS staging of a ROWS x D bf16 tile by NT threads.  load() issues all the
 // global loads of the thread back to back (rows past the end are clamped to the last valid row so
 // that the loads need no branches; their data is zeroed in store()), store() writes them to LDS.

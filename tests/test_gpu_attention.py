@@ -195,3 +195,26 @@ def test_full_size_properties_and_slice(gpu, name):
     starts = (wl.position_ids == 0)
     for h in (0, sp.Hq - 1):
         assert torch.equal(out[:, :, h][starts], wl.xv[:, :, h // G][starts])
+
+
+@pytest.mark.parametrize("heads", [(2, 1), (4, 2), (2, 2)], ids=["pair_g2", "pair_g2_hkv2", "single_g1"])
+@pytest.mark.parametrize("D", [128, 256])
+def test_bf16_forward_scores_that_outgrow_the_first_block(gpu, heads, D):
+    """Late keys score far above anything in a row's first kv block (hundreds of nats): the online
+    softmax must move its reference (rescale, or redo the tile in two passes) and stay exact."""
+    Hq, Hkv = heads
+    B, S = 1, 640
+    q, k, v, _ = _qkv(B, S, Hq, Hkv, D, torch.bfloat16, 11)
+    k = k.clone()
+    k[:, 300:] *= 60.0          # logits of late keys have std 60 instead of 1
+    k[:, 500:] *= 4.0           # and grow once more
+    ids = _ids(B, S, 3, "docs")
+    ids[:] = 0                  # one document: every row sees all earlier keys
+    scale = D ** -0.5
+    want, wl = A.dense_attention(q, k, v, ids, scale, True, None, return_lse=True)
+    gids = ids.to(gpu)
+    tm = build_tile_map(gids, B, S, True, None, device=gpu)
+    out, lse = attention_forward(q.to(gpu), k.to(gpu), v.to(gpu), tm, gids, scale, True, None)
+    _check(out, want, torch.bfloat16, ("outgrown", heads, D))
+    assert torch.isfinite(lse).all()
+    assert max_abs(lse.cpu(), wl) <= 2e-2 * max(1.0, float(wl.abs().max()) / 100)
