@@ -27,8 +27,12 @@ namespace ma {
 
 constexpr int kPairThreads = 256;
 constexpr int kPairBN = 64;   // kv rows staged per step
-constexpr int kPairPipeK = 3;
-constexpr int kPairPipeV = 3;
+#ifndef MA_PAIR_PK
+#define MA_PAIR_PK 2
+#define MA_PAIR_PV 2
+#endif
+constexpr int kPairPipeK = MA_PAIR_PK;  // LDS fragment reads in flight ahead of the MFMAs (registers are tight)
+constexpr int kPairPipeV = MA_PAIR_PV;
 
 template <int D, bool HAS_DOC>
 __global__ __launch_bounds__(kPairThreads) void attn_fwd_pair_bf16_kernel(AttnArgs a) {
