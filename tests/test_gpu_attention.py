@@ -9,7 +9,7 @@ import torch
 
 from conftest import max_abs, rel_l2
 from maester_amd import build_tile_map, doc_masked_attention, packed_doc_attention, workloads
-from maester_amd.attention import attention_forward
+from maester_amd.attention import attention_backward, attention_forward
 from oracle import attention as A
 from oracle import prologue as P
 
@@ -195,6 +195,30 @@ def test_full_size_properties_and_slice(gpu, name):
     starts = (wl.position_ids == 0)
     for h in (0, sp.Hq - 1):
         assert torch.equal(out[:, :, h][starts], wl.xv[:, :, h // G][starts])
+
+
+@pytest.mark.parametrize("name", ["c2", "c3", "c4", "c5"])
+def test_full_size_backward_slices(gpu, name):
+    """At the benchmark shapes: forward and backward of the whole batch through the C ABI, then two
+    (row, kv head) slices of out / dq / dk / dv against the fp32 oracle evaluated on the GPU (the
+    dense score matrix of one slice is all that fits)."""
+    wl = workloads.make(name).to(gpu)
+    sp = wl.spec
+    q, k, v, do = wl.xq, wl.xk, wl.xv, wl.dout
+    tm = build_tile_map(wl.document_ids, sp.B, sp.S, True, sp.window)
+    out, lse = attention_forward(q, k, v, tm, wl.document_ids, wl.scale, True, sp.window)
+    dq, dk, dv = attention_backward(q, k, v, out, do, lse, tm, wl.document_ids, wl.scale, True, sp.window)
+    G = sp.Hq // sp.Hkv
+    for b, hk in ((0, 0), (sp.B - 1, sp.Hkv - 1)):
+        hs = slice(hk * G, (hk + 1) * G)
+        ids = wl.document_ids[b:b + 1]
+        wo, wq, wk, wv = A.dense_attention_fwd_bwd(q[b:b + 1, :, hs], k[b:b + 1, :, hk:hk + 1], v[b:b + 1, :, hk:hk + 1],
+                                                   do[b:b + 1, :, hs], ids, wl.scale, True, sp.window)
+        for what, got, want in (("out", out[b:b + 1, :, hs], wo), ("dq", dq[b:b + 1, :, hs], wq),
+                                ("dk", dk[b:b + 1, :, hk:hk + 1], wk), ("dv", dv[b:b + 1, :, hk:hk + 1], wv)):
+            _check(got.cpu(), want.cpu(), torch.bfloat16, (name, b, hk, what))
+        del wo, wq, wk, wv
+        torch.cuda.empty_cache()
 
 
 @pytest.mark.parametrize("heads", [(2, 1), (4, 2), (2, 2)], ids=["pair_g2", "pair_g2_hkv2", "single_g1"])
