@@ -370,70 +370,8 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dq_bf16_kernel(AttnArgs 
     const bool own_delta = (a.stages & MA_BWD_DELTA) != 0;
     float delta = own_delta ? 0.f : a.delta[rowi];
 
-    // Q and dO rows of the workgroup come in through LDS (coalesced) and stay in registers (AGPRs)
-    bf16x8 qf[KK], gf[KK];
-    {
-        DirectStager<D, kTile, NW> sq;
-        sq.init(w, lane);
-        const int rows_valid = min(kTile, a.S - i * kTile);
-        sq.issue(qp + (int64_t)i * kTile * a.q.stride_s, Kbuf(0), w, lane, rows_valid, a.q.stride_s);
-        sq.issue(gp + (int64_t)i * kTile * a.dout.stride_s, Kbuf(1), w, lane, rows_valid, a.dout.stride_s);
-        // the wave's O rows go straight to registers, whole rows per load (coalesced); they meet the
-        // dO rows, read back from the LDS tile in the same row-major order, in delta's dot products
-        constexpr int CH = D / 8, RPI = 64 / CH, NIT = 32 / RPI;  // 16-byte chunks per row, rows per load, loads
-        const int orow = lane / CH, oc = lane % CH;
-        u32x4 ov[NIT];
-        if (own_delta) {
-            const __bf16* obase = (const __bf16*)a.o.ptr + b * a.o.stride_b + h * a.o.stride_h + oc * 8;
-#pragma unroll
-            for (int it = 0; it < NIT; ++it)
-                ov[it] = *(const u32x4*)(obase + (int64_t)min(qw_lo + it * RPI + orow, a.S - 1) * a.o.stride_s);
-        }
-        wait_vmem();
-        __syncthreads();
-#pragma unroll
-        for (int kk = 0; kk < KK; ++kk) {
-            qf[kk] = TL::row_frag(Kbuf(0), rbase, 32 * w, kk);
-            gf[kk] = TL::row_frag(Kbuf(1), rbase, 32 * w, kk);
-        }
-        if (own_delta) {
-            // partial dot product per (row, chunk) -> per-wave LDS scratch [32 rows][CH] -> row sums
-            MA_LDS float* part = (MA_LDS float*)(lds0 + 4 * TL::bytes(BN) + 2 * BN * 8) + w * 32 * CH;
-#pragma unroll
-            for (int it = 0; it < NIT; ++it) {
-                const int row = it * RPI + orow;
-                const u32x4 g = *(MA_LDS u32x4*)(Kbuf(1) + TL::off(32 * w + row, oc * 8));
-                float acc = 0.f;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {  // bf16 -> fp32 is a 16-bit shift
-                    acc += __builtin_bit_cast(float, ov[it][e] << 16) * __builtin_bit_cast(float, g[e] << 16);
-                    acc += __builtin_bit_cast(float, ov[it][e] & 0xffff0000u) * __builtin_bit_cast(float, g[e] & 0xffff0000u);
-                }
-                part[row * CH + oc] = acc;
-            }
-            // lane (r, hh) sums half of row r's chunks; the other half comes from lane (r, 1 - hh)
-            float sum = 0.f;
-#pragma unroll
-            for (int c4 = 0; c4 < CH / 8; ++c4) {
-                const f32x4 p4 = *(MA_LDS f32x4*)(part + r * CH + hh * (CH / 2) + 4 * c4);
-                sum += (p4[0] + p4[1]) + (p4[2] + p4[3]);
-            }
-            delta = sum + xor32(sum);
-            if (qvalid && hh == 0) a.delta[rowi] = delta;
-        }
-        // From here on the fragments are MFMA operands only: move them to AGPRs once, now.  (Left to
-        // the register allocator, fragments that were also read by the vector ALU stay in VGPRs and
-        // get copied to AGPRs right in front of every MFMA that uses them.)
-        static_for<0, KK>([&](auto kk) { park_in_agprs(qf[decltype(kk)::value], gf[decltype(kk)::value]); });
-        __syncthreads();
-    }
-
-    f32x16 acc[DB];
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) acc[db][v] = 0.f;
-
+    // The walk over the kv tiles is set up first: its index loads are then ahead of the bulk loads
+    // below in the memory pipeline, and the first K/V tiles can be requested as soon as they return.
     const size_t mrow = (size_t)b * a.T + i;
     const bool windowed = a.window >= 0;
     StepWalk<BN> st;
@@ -448,11 +386,40 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dq_bf16_kernel(AttnArgs 
     // document-id ranges: of the wave's own q rows now, of the two kv blocks of a step at each step
     const bool use_rng = HAS_DOC && a.map.block_doc_range != nullptr;
     const int64_t* rng_row = use_rng ? a.map.block_doc_range + (size_t)b * (2 * ((a.S + 63) / 64)) * 2 : nullptr;
+
+    // Q and dO rows of the wave go straight from global memory into MFMA operand fragments: lane
+    // (r, hh) holds elements 16*kk + 8*hh .. +7 of row qw_lo + r, one 16-byte load each (the two
+    // halves of a wave read adjacent 16 bytes, every 128-byte line is used in full by four loads).
+    // Nothing passes through LDS, so the index lists and the first K/V tiles are fetched at the
+    // same time instead of after a barrier.
+    bf16x8 qf[KK], gf[KK];
+    u32x4 of[KK];
+    {
+        const __bf16* qrow = qp + (int64_t)qc * a.q.stride_s + 8 * hh;
+        const __bf16* grow = gp + (int64_t)qc * a.dout.stride_s + 8 * hh;
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) qf[kk] = *(const bf16x8*)(qrow + 16 * kk);
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) gf[kk] = *(const bf16x8*)(grow + 16 * kk);
+        if (own_delta) {
+            const __bf16* orow = (const __bf16*)a.o.ptr + b * a.o.stride_b + h * a.o.stride_h + (int64_t)qc * a.o.stride_s + 8 * hh;
+#pragma unroll
+            for (int kk = 0; kk < KK; ++kk) of[kk] = *(const u32x4*)(orow + 16 * kk);
+        }
+    }
+
+    // (load and wait stay adjacent: the registers of a scalar load in flight must not be touched)
     DocRange own;
     if (use_rng) {
         own.load(rng_row + (size_t)(min(qw_lo, a.S - 1) / MA_DOC_BLOCK) * 2);
         own.ready();
     }
+
+    f32x16 acc[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[db][v] = 0.f;
 
     DirectStager<D, BN, NW> sk;  // the K and V tiles have the same shape: one set of slots
     sk.init(w, lane);
@@ -477,6 +444,26 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dq_bf16_kernel(AttnArgs 
         issue_v(0);
         issue_ids();
     }
+
+    if (own_delta) {
+        // lane (r, hh) sums its half of row r's products; the other half is in lane (r, 1 - hh)
+        float sum = 0.f;
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+            const u32x4 g = __builtin_bit_cast(u32x4, gf[kk]);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {  // bf16 -> fp32 is a 16-bit shift
+                sum += __builtin_bit_cast(float, of[kk][e] << 16) * __builtin_bit_cast(float, g[e] << 16);
+                sum += __builtin_bit_cast(float, of[kk][e] & 0xffff0000u) * __builtin_bit_cast(float, g[e] & 0xffff0000u);
+            }
+        }
+        delta = sum + xor32(sum);
+        if (qvalid && hh == 0) a.delta[rowi] = delta;
+    }
+    // From here on the fragments are MFMA operands only: move them to AGPRs once, now.  (Left to
+    // the register allocator, fragments that were also read by the vector ALU stay in VGPRs and
+    // get copied to AGPRs right in front of every MFMA that uses them.)
+    static_for<0, KK>([&](auto kk) { park_in_agprs(qf[decltype(kk)::value], gf[decltype(kk)::value]); });
 
     for (int n = 0; have; ++n) {
         const int cur = n & 1;
@@ -601,8 +588,7 @@ static int bwd_dd(const AttnArgs& a, hipStream_t st) {
         if (rc) return rc;
     }
     if (a.stages & MA_BWD_DQ) {  // first: the dK/dV kernel reads the delta this one may be writing
-        // K/V ring, kv document ids, and the per-wave scratch of the delta row sums
-        const size_t lds_q = (size_t)4 * Tile<D>::bytes(kStep) + 2 * kStep * 8 + (size_t)(kBwdThreads / 64) * 32 * (D / 8) * 4;
+        const size_t lds_q = (size_t)4 * Tile<D>::bytes(kStep) + 2 * kStep * 8;  // K/V ring, kv document ids
         rc = opt_in_lds(attn_bwd_dq_bf16_kernel<D, HAS_DOC>, lds_q, "attn_bwd_dq_bf16");
         if (rc) return rc;
         hipLaunchKernelGGL((attn_bwd_dq_bf16_kernel<D, HAS_DOC>), dim3(work_grid(a.B * a.T, a.Hkv, a.Hq / a.Hkv), 1, 1), dim3(kBwdThreads),

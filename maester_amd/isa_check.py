@@ -1,0 +1,122 @@
+"""Static checks of the compiler's output for the kernels that issue instructions through ``asm``.
+
+The compiler knows nothing about what an ``asm`` statement does, so two kinds of hazard that it
+normally handles are the source's responsibility there; this module re-checks them on the generated
+gfx950 assembly (``python -m maester_amd.isa_check`` or ``check_all()``):
+
+1. **MFMA results.**  No hazard padding is inserted around ``asm`` MFMAs: between an MFMA and the
+   next fence (``s_nop`` of 16 wait states), branch, label or barrier, no compiler-scheduled vector
+   or memory instruction may read or write a register that an MFMA of the current chain writes.
+2. **Scalar loads in flight.**  An ``asm`` ``s_load`` returns its data some hundred cycles later,
+   into the physical registers it named.  Until the next ``s_waitcnt lgkmcnt(0)`` nothing may read
+   or write those registers: a spill of the (not yet loaded) tuple, followed by a reuse of the
+   registers for something else, ends with the load overwriting that something else.
+"""
+from __future__ import annotations
+
+import os
+import re
+import subprocess
+import sys
+import tempfile
+from concurrent.futures import ThreadPoolExecutor
+
+CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
+SOURCES = ["attn_fwd_bf16.hip", "attn_fwd_pair_bf16.hip", "attn_bwd_bf16.hip"]
+FLAGS = ("--offload-arch=gfx950 -O3 -std=c++17 -ffast-math -fno-finite-math-only -Xclang -target-feature "
+         "-Xclang -packed-fp32-ops -S --cuda-device-only").split()
+
+
+def _regs(text: str, classes: str) -> set:
+    """(class, index) of every register of the given classes named in an operand string."""
+    out = set()
+    for cls, lo, hi in re.findall(r"\b([%s])\[(\d+):(\d+)\]" % classes, text):
+        out |= {(cls, i) for i in range(int(lo), int(hi) + 1)}
+    for cls, i in re.findall(r"\b([%s])(\d+)\b" % classes, text):
+        out.add((cls, int(i)))
+    return out
+
+
+def check_assembly(asm: str) -> tuple[list[str], dict]:
+    """Returns (violations, {kernel: (asm MFMAs, asm scalar loads)})."""
+    bad, stats = [], {}
+    for m in re.finditer(r"^(_ZN2ma\w+):[^\n]*\n(.*?)s_endpgm", asm, re.S | re.M):
+        name, body = m.group(1), m.group(2).split("\n")
+        in_asm = False
+        chain = set()      # vector registers written by MFMAs of the current chain
+        pending = set()    # scalar registers of asm loads that have not been waited for
+        n_mfma = n_sload = 0
+        for i, ln in enumerate(body):
+            t = ln.strip()
+            if t.startswith(";;#ASMSTART"):
+                in_asm = True
+                continue
+            if t.startswith(";;#ASMEND"):
+                in_asm = False
+                continue
+            if not t or t.startswith(";"):
+                continue
+            if t.startswith((".LBB", "s_cbranch", "s_branch", "s_barrier")):
+                chain = set()
+                if pending and t.startswith(("s_cbranch", "s_branch")):
+                    # a branch between an asm load and its wait: the linear scan no longer follows the program
+                    pass
+                continue
+            mm = re.match(r"s_nop (\d+)", t)
+            if mm:
+                if int(mm.group(1)) >= 15:
+                    chain = set()
+                continue
+            ops = t.split(None, 1)[1] if " " in t else ""
+            if t.startswith("s_waitcnt"):
+                if "lgkmcnt(0)" in t:
+                    pending = set()
+                continue
+            if pending:
+                hit = _regs(ops, "s") & pending
+                if hit and not (in_asm and t.startswith("s_load")):
+                    bad.append(f"{name} line {i}: '{t}' touches scalar registers of a load in flight {sorted(hit)[:4]}")
+            if in_asm:
+                if t.startswith("v_mfma"):
+                    n_mfma += 1
+                    chain |= _regs(ops.split(",")[0], "va")
+                elif t.startswith("s_load"):
+                    n_sload += 1
+                    pending |= _regs(ops.split(",")[0], "s")
+                continue
+            if chain and re.match(r"(v_|ds_|global_|buffer_|flat_|scratch_)", t):
+                hit = _regs(ops, "va") & chain
+                if hit:
+                    bad.append(f"{name} line {i}: '{t}' touches in-flight MFMA result {sorted(hit)[:4]}")
+        stats[name] = (n_mfma, n_sload)
+    return bad, stats
+
+
+def compile_to_assembly(source: str) -> str:
+    with tempfile.TemporaryDirectory() as tmp:
+        out = os.path.join(tmp, "k.s")
+        r = subprocess.run(["hipcc", *FLAGS, os.path.join(CSRC, source), "-o", out], capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError(f"hipcc -S {source} failed:\n{r.stderr[-2000:]}")
+        with open(out) as f:
+            return f.read()
+
+
+def check_all(sources=SOURCES) -> tuple[list[str], dict]:
+    bad, stats = [], {}
+    with ThreadPoolExecutor(max_workers=len(sources)) as pool:
+        for asm in pool.map(compile_to_assembly, sources):
+            b, s = check_assembly(asm)
+            bad += b
+            stats.update(s)
+    return bad, stats
+
+
+if __name__ == "__main__":
+    bad, stats = check_all(sys.argv[1:] or SOURCES)
+    for name, (nm, ns) in stats.items():
+        print(f"{name}: {nm} asm MFMAs, {ns} asm scalar loads")
+    for b in bad[:40]:
+        print(b)
+    print("BAD" if bad else "OK")
+    sys.exit(1 if bad else 0)

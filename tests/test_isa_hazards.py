@@ -1,0 +1,41 @@
+"""The hazards that `asm` statements hide from the compiler, re-checked on the generated gfx950
+assembly (no GPU needed: hipcc cross-compiles)."""
+import shutil
+
+import pytest
+
+from maester_amd import isa_check
+
+FAULTY = """
+_ZN2ma4demoEv: ; @demo
+	;;#ASMSTART
+	s_load_dwordx4 s[52:55], s[2:3], 0x0
+	;;#ASMEND
+	v_writelane_b32 v170, s52, 9
+	;;#ASMSTART
+	s_waitcnt lgkmcnt(0)
+	;;#ASMEND
+	;;#ASMSTART
+	v_mfma_f32_32x32x16_bf16 v[0:15], v[16:19], a[0:3], v[0:15]
+	;;#ASMEND
+	v_add_f32_e32 v1, v1, v20
+	s_endpgm
+"""
+
+
+def test_checker_flags_both_kinds_of_hazard():
+    bad, stats = isa_check.check_assembly(FAULTY)
+    assert stats == {"_ZN2ma4demoEv": (1, 1)}
+    assert len(bad) == 2 and "load in flight" in bad[0] and "MFMA result" in bad[1]
+    clean = FAULTY.replace("\tv_writelane_b32 v170, s52, 9\n", "").replace("\tv_add_f32_e32 v1, v1, v20\n", "\ts_nop 15\n\tv_add_f32_e32 v1, v1, v20\n")
+    assert isa_check.check_assembly(clean)[0] == []
+
+
+@pytest.mark.skipif(shutil.which("hipcc") is None, reason="hipcc not installed")
+def test_generated_assembly_of_the_attention_kernels_is_hazard_free():
+    bad, stats = isa_check.check_all()
+    assert not bad, "\n".join(bad[:20])
+    # every bf16 attention kernel went through the checker, and its asm MFMAs were seen
+    for kernel in ("attn_fwd_bf16_kernel", "attn_fwd_pair_bf16_kernel", "attn_bwd_dq_bf16_kernel", "attn_bwd_dkv_bf16_kernel"):
+        hits = [v for k, v in stats.items() if kernel in k]
+        assert len(hits) == 6 and all(n_mfma > 0 for n_mfma, _ in hits), (kernel, hits)
