@@ -153,8 +153,9 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dkv_bf16_kernel(AttnArgs
     {
         int lo, hi;
         visibility_limits(true, j * kTile, j * kTile + kTile - 1, BM, bounded, wlim, windowed, lo, hi);
-        st.init(a.map.q_indices + mrow * a.T, a.map.q_num_blocks[mrow], a.map.full_q_indices + mrow * a.T,
-                a.map.full_q_num_blocks[mrow], G, true, a.S, lo, hi);
+        int n_partial, n_full;
+        scalar_load2(a.map.q_num_blocks + mrow, a.map.full_q_num_blocks + mrow, n_partial, n_full);
+        st.init(a.map.q_indices + mrow * a.T, n_partial, a.map.full_q_indices + mrow * a.T, n_full, G, true, a.S, lo, hi);
     }
     int blk_lo, blk_hi;
     visibility_limits(true, kw_lo, kw_hi, 32, bounded, wlim, windowed, blk_lo, blk_hi);
@@ -194,7 +195,7 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dkv_bf16_kernel(AttnArgs
     auto issue_q = [&](int buf) { sq.issue((const __bf16*)qsrc, Qbuf(buf), w, lane, min(BM, a.S - st.r0), a.q.stride_s); };
     auto issue_g = [&](int buf) { sq.issue((const __bf16*)gsrc, Gbuf(buf), w, lane, min(BM, a.S - st.r0), a.dout.stride_s); };
     const int my_runs = decltype(sq)::runs_of(w);
-    bool have = st.next();
+    bool have = st.first();
     int q0 = st.r0;
     bool partial = st.partial;
     if (have) {
@@ -378,8 +379,9 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dq_bf16_kernel(AttnArgs 
     {
         int lo, hi;
         visibility_limits(false, i * kTile, i * kTile + kTile - 1, BN, bounded, wlim, windowed, lo, hi);
-        st.init(a.map.kv_indices + mrow * a.T, a.map.kv_num_blocks[mrow], a.map.full_kv_indices + mrow * a.T,
-                a.map.full_kv_num_blocks[mrow], 1, false, a.S, lo, hi);
+        int n_partial, n_full;
+        scalar_load2(a.map.kv_num_blocks + mrow, a.map.full_kv_num_blocks + mrow, n_partial, n_full);
+        st.init(a.map.kv_indices + mrow * a.T, n_partial, a.map.full_kv_indices + mrow * a.T, n_full, 1, false, a.S, lo, hi);
     }
     int blk_lo, blk_hi;
     visibility_limits(false, qw_lo, qw_hi, 32, bounded, wlim, windowed, blk_lo, blk_hi);
@@ -436,7 +438,7 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dq_bf16_kernel(AttnArgs 
         if (HAS_DOC && st.partial && tid < BN) kd_next = drow[min(st.r0 + tid, a.S - 1)];
     };
     const int my_runs = decltype(sk)::runs_of(w);
-    bool have = st.next();
+    bool have = st.first();
     int k0 = st.r0;
     bool partial = st.partial;
     if (have) {

@@ -84,8 +84,9 @@ __global__ __launch_bounds__(kFwdThreads) void attn_fwd_bf16_kernel(AttnArgs a) 
     {
         int lo, hi;
         visibility_limits(false, i * kTile, i * kTile + kTile - 1, BN, bounded, wlim, windowed, lo, hi);
-        st.init(a.map.kv_indices + mrow * a.T, a.map.kv_num_blocks[mrow], a.map.full_kv_indices + mrow * a.T,
-                a.map.full_kv_num_blocks[mrow], 1, false, a.S, lo, hi);
+        int n_partial, n_full;
+        scalar_load2(a.map.kv_num_blocks + mrow, a.map.full_kv_num_blocks + mrow, n_partial, n_full);
+        st.init(a.map.kv_indices + mrow * a.T, n_partial, a.map.full_kv_indices + mrow * a.T, n_full, 1, false, a.S, lo, hi);
     }
     int blk_lo, blk_hi;
     visibility_limits(false, qw_lo, qw_hi, 32, bounded, wlim, windowed, blk_lo, blk_hi);
@@ -102,7 +103,7 @@ __global__ __launch_bounds__(kFwdThreads) void attn_fwd_bf16_kernel(AttnArgs a) 
     sk.init(w, lane);
     int64_t kd_next = 0;
     const int my_runs = decltype(sk)::runs_of(w);
-    bool have = st.next();
+    bool have = st.first();
     int k0 = st.r0;
     bool partial = st.partial;
     if (have) {

@@ -67,16 +67,6 @@ __global__ __launch_bounds__(kPairThreads) void attn_fwd_pair_bf16_kernel(AttnAr
     const int64_t* drow = HAS_DOC ? a.doc + (size_t)b * a.S : nullptr;
     const int rbase = TL::row_base(lane), tbase = TL::tr_base(lane);
 
-    // Both heads' Q tiles come in through LDS (coalesced), one per K/V buffer pair, and stay in VGPRs.
-    bf16x8 qa[KK], qb[KK];
-    {
-        DirectStager<D, kTile, NW> sq;
-        sq.init(w, lane);
-        const int rows_valid = min(kTile, a.S - i * kTile);
-        sq.issue(qp + (int64_t)i * kTile * a.q.stride_s, Kbuf(0), w, lane, rows_valid, a.q.stride_s);
-        sq.issue(qp + a.q.stride_h + (int64_t)i * kTile * a.q.stride_s, Kbuf(1), w, lane, rows_valid, a.q.stride_s);
-    }
-
     const int qc = min(q, a.S - 1);
     const int64_t docq = HAS_DOC ? drow[qc] : 0;
     const bool windowed = a.window >= 0;
@@ -100,14 +90,41 @@ __global__ __launch_bounds__(kPairThreads) void attn_fwd_pair_bf16_kernel(AttnAr
     const int my_runs = decltype(sk)::runs_of(w);
     int64_t kd_next = 0;
 
-    wait_vmem();
-    __syncthreads();
+    // The walk over the kv tiles: its index loads go out first, then both heads' Q rows, which go
+    // straight from global memory into MFMA operand fragments (lane (r, hh): elements 16*kk + 8*hh
+    // .. +7 of row qw_lo + r, one 16-byte load each; nothing passes through LDS), then, once the
+    // index loads are back, the first K/V tiles -- all in flight together.
+    bool have;
+    int k0;
+    bool partial;
+    auto walk_init = [&]() {
+        int lo, hi;
+        visibility_limits(false, i * kTile, i * kTile + kTile - 1, BN, bounded, wlim, windowed, lo, hi);
+        int n_partial, n_full;
+        scalar_load2(a.map.kv_num_blocks + mrow, a.map.full_kv_num_blocks + mrow, n_partial, n_full);
+        st.init(a.map.kv_indices + mrow * a.T, n_partial, a.map.full_kv_indices + mrow * a.T, n_full, 1, false, a.S, lo, hi);
+    };
+    auto walk_first = [&]() {
+        have = st.first();
+        k0 = st.r0;
+        partial = st.partial;
+        if (have) {
+            const int rows_valid = min(BN, a.S - k0);
+            sk.issue((const __bf16*)(kp + (uint64_t)(uint32_t)k0 * ksb), Kbuf(0), w, lane, rows_valid, a.k.stride_s);
+            sk.issue((const __bf16*)(vp + (uint64_t)(uint32_t)k0 * vsb), Vbuf(0), w, lane, rows_valid, a.v.stride_s);
+            if (HAS_DOC && partial && tid < BN) kd_next = drow[min(k0 + tid, a.S - 1)];
+        }
+    };
+    walk_init();
+    bf16x8 qa[KK], qb[KK];
+    {
+        const __bf16* qrow = qp + (int64_t)qc * a.q.stride_s + 8 * hh;
 #pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-        qa[kk] = TL::row_frag(Kbuf(0), rbase, 32 * w, kk);
-        qb[kk] = TL::row_frag(Kbuf(1), rbase, 32 * w, kk);
+        for (int kk = 0; kk < KK; ++kk) qa[kk] = *(const bf16x8*)(qrow + 16 * kk);
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) qb[kk] = *(const bf16x8*)(qrow + a.q.stride_h + 16 * kk);
     }
-    __syncthreads();  // all Q fragments are in registers before the buffers are reused
+    walk_first();
 
     // O^T of both heads: all 256 AGPRs (D = 256); nothing but MFMAs touches them inside the loop
     f32x16 oa[DB], ob[DB];
@@ -126,20 +143,9 @@ __global__ __launch_bounds__(kPairThreads) void attn_fwd_pair_bf16_kernel(AttnAr
     pin_tiles<0, DB, true>(ob);
     la = lb = 0.f;
     if (mode != 2) ma_ = mb_ = -INFINITY;
-    {
-        int lo, hi;
-        visibility_limits(false, i * kTile, i * kTile + kTile - 1, BN, bounded, wlim, windowed, lo, hi);
-        st.init(a.map.kv_indices + mrow * a.T, a.map.kv_num_blocks[mrow], a.map.full_kv_indices + mrow * a.T,
-                a.map.full_kv_num_blocks[mrow], 1, false, a.S, lo, hi);
-    }
-    bool have = st.next();
-    int k0 = st.r0;
-    bool partial = st.partial;
-    if (have) {
-        const int rows_valid = min(BN, a.S - k0);
-        sk.issue((const __bf16*)(kp + (uint64_t)(uint32_t)k0 * ksb), Kbuf(0), w, lane, rows_valid, a.k.stride_s);
-        sk.issue((const __bf16*)(vp + (uint64_t)(uint32_t)k0 * vsb), Vbuf(0), w, lane, rows_valid, a.v.stride_s);
-        if (HAS_DOC && partial && tid < BN) kd_next = drow[min(k0 + tid, a.S - 1)];
+    if (mode) {  // a later pass starts the walk again
+        walk_init();
+        walk_first();
     }
 
     for (int n = 0; have; ++n) {

@@ -62,6 +62,21 @@ int launch_attn_fwd_bf16(const AttnArgs& a, hipStream_t st);
 int launch_attn_fwd_pair_bf16(const AttnArgs& a, hipStream_t st);  // even number of q heads per kv head
 int launch_attn_bwd_bf16(const AttnArgs& a, hipStream_t st);
 
+// Loads through the scalar cache, waited for on the spot.  For the handful of uniform values a
+// workgroup needs before it can request its first tiles: a scalar load has a fraction of a vector
+// load's latency and its wait (lgkmcnt) does not queue behind the bulk vector loads already in
+// flight.  Load and wait are one asm statement, so the compiler cannot touch the destination
+// registers in between.
+__device__ __forceinline__ int scalar_load(const int32_t* p) {
+    int v;
+    asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(v) : "s"(p) : "memory");
+    return v;
+}
+__device__ __forceinline__ void scalar_load2(const int32_t* p, const int32_t* q, int& a, int& b) {
+    asm volatile("s_load_dword %0, %2, 0x0\n\ts_load_dword %1, %3, 0x0\n\ts_waitcnt lgkmcnt(0)"
+                 : "=&s"(a), "=&s"(b) : "s"(p), "s"(q) : "memory");
+}
+
 // Workgroup id -> work item.  A unit is a tile row (q tile for the forward and dQ kernels, kv tile
 // for the dK/dV kernel) of one batch row; a combo is (unit, kv head) and owns `heads` workgroups
 // (the query heads that stream the same K/V, or 1).  Workgroups are handed to the 8 XCDs round-robin
@@ -80,10 +95,12 @@ __device__ __forceinline__ bool map_work(int id, int n_units, int T, int Hkv, in
     const int c = (n / heads) * kXcds + x;
     if (c >= n_units * Hkv) return false;
     const int rank = c / Hkv, hk = c % Hkv;
-    const int u = order ? order[rank] : rank;
-    b = u / T;
-    tile = u % T;
-    head = hk * heads + g;
+    const int u = order ? scalar_load(order + __builtin_amdgcn_readfirstlane(rank)) : rank;
+    // (integer division runs on the vector ALU: hand the results back as scalars, so that everything
+    // derived from them -- tile-map rows, base pointers -- is addressed and loaded on the scalar side)
+    b = __builtin_amdgcn_readfirstlane(u / T);
+    tile = __builtin_amdgcn_readfirstlane(u % T);
+    head = __builtin_amdgcn_readfirstlane(hk * heads + g);
     return true;
 }
 
@@ -105,10 +122,27 @@ struct ListWalk {
         return i < np ? pl[i + zero] : fl[i - np + zero];
     }
     __device__ __forceinline__ void init(const int32_t* partial_list, int n_partial, const int32_t* full_list, int n_full,
-                                         int repeats, bool reverse, int zero) {
+                                         int repeats, bool reverse) {
         pl = partial_list; fl = full_list; np = n_partial; n = n_partial + n_full; reps = repeats;
         rep = 0; it = -1; backward = reverse;
-        nxt = n ? fetch(0, zero) : 0;
+        nxt = 0;
+    }
+    // The start of a walk: the entry is loaded and waited for on the spot (uniform address: a scalar
+    // load, whose wait does not queue behind the bulk vector loads a kernel has in flight when it
+    // starts) -- advance_now() until the first step is found, then prefetch() once; advance() from then on.
+    __device__ __forceinline__ bool advance_now(int& tile, bool& partial) {
+        if (n == 0) return false;
+        if (++it == n) {
+            it = 0;
+            if (++rep == reps) return false;
+        }
+        const int i = backward ? n - 1 - it : it;
+        tile = scalar_load(i < np ? pl + i : fl + (i - np));
+        partial = (backward ? n - 1 - it : it) < np;
+        return true;
+    }
+    __device__ __forceinline__ void prefetch(int zero) {
+        if (n) nxt = fetch(it + 1 == n ? 0 : it + 1, zero);
     }
     __device__ __forceinline__ bool advance(int& tile, bool& partial, int zero) {
         if (n == 0) return false;
@@ -137,13 +171,27 @@ struct StepWalk {
     __device__ __forceinline__ void init(const int32_t* partial_list, int n_partial, const int32_t* full_list, int n_full,
                                          int repeats, bool reverse, int seq_len, int lo, int hi) {
         zero = opaque_lane_zero_();
-        walk.init(partial_list, n_partial, full_list, n_full, repeats, reverse, zero);
+        walk.init(partial_list, n_partial, full_list, n_full, repeats, reverse);
         half = kTile / STEP - 1; tile = 0; partial = false; S = seq_len; vis_lo = lo; vis_hi = hi; r0 = 0;
     }
     __device__ __forceinline__ static int opaque_lane_zero_() {
         int z;
         asm volatile("v_mov_b32 %0, 0" : "=v"(z));
         return z;
+    }
+    // the first step of the walk (see ListWalk::advance_now), then next() for the others
+    __device__ __forceinline__ bool first() {
+        for (;;) {
+            if (++half == kTile / STEP) {
+                half = 0;
+                if (!walk.advance_now(tile, partial)) return false;
+            }
+            r0 = tile * kTile + half * STEP;
+            if ((r0 < S) & (!partial | ((r0 >= vis_lo) & (r0 <= vis_hi)))) {
+                walk.prefetch(zero);
+                return true;
+            }
+        }
     }
     __device__ __forceinline__ bool next() {
         for (;;) {
