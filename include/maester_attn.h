@@ -38,6 +38,7 @@ extern "C" {
 
 #define MA_TILE 128 /* BlockMask tile edge (torch _DEFAULT_SPARSE_BLOCK_SIZE) */
 #define MA_DOC_BLOCK 32 /* rows per entry of ma_tile_map.block_doc_range */
+#define MA_WORK_COUNTERS 64 /* ints in ma_tile_map.work_counters */
 
 /* Library version (major*10000 + minor*100 + patch). */
 int ma_version(void);
@@ -72,6 +73,14 @@ typedef struct ma_tile_map {
      * and kv rows have disjoint id ranges -- no pair of them can share a document.  May be NULL, and
      * is ignored when document_ids is NULL (then nothing is skipped on that ground). */
     int64_t* block_doc_range;    /* [B, 2 * ceil(S / 64), 2]: blocks past the end repeat the last row */
+    /* Work queues of the attention kernels (not part of BlockMask): MA_WORK_COUNTERS ints that
+     * ma_tile_map_build zeroes.  With it, a kernel is launched as one workgroup per compute unit and
+     * the workgroups pull work items (in the order of the launch schedules) until none is left, which
+     * keeps every compute unit busy to the end; the last workgroup of a launch puts the counters back
+     * to zero.  Launches that share a tile map must therefore be ordered (same stream, or events):
+     * two of them running at once would share the counters.  May be NULL: then one workgroup is
+     * launched per work item, as many as there are, and the hardware dispatcher places them. */
+    int32_t* work_counters;      /* [MA_WORK_COUNTERS] */
 } ma_tile_map;
 
 /* ---- block-sparse tile map --------------------------------------------------------------------

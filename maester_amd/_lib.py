@@ -21,6 +21,7 @@ MA_DTYPE_F32 = 0
 MA_DTYPE_BF16 = 1
 MA_TILE = 128
 MA_DOC_BLOCK = 32
+MA_WORK_COUNTERS = 64
 MA_BWD_DELTA, MA_BWD_DKV, MA_BWD_DQ, MA_BWD_ALL = 1, 2, 4, 7
 
 EXPORTS = (
@@ -38,7 +39,7 @@ class MaTileMap(Structure):
     _fields_ = [(n, c_void_p) for n in (
         "kv_num_blocks", "kv_indices", "full_kv_num_blocks", "full_kv_indices",
         "q_num_blocks", "q_indices", "full_q_num_blocks", "full_q_indices", "q_tile_order", "kv_tile_order",
-        "block_doc_range")]
+        "block_doc_range", "work_counters")]
 
 
 class MaesterAttnError(RuntimeError):

@@ -84,7 +84,7 @@ __global__ __launch_bounds__(256) void attn_delta_bf16_kernel(AttnArgs a) {
 // dK / dV
 // ------------------------------------------------------------------------------------------------
 template <int D, bool HAS_DOC>
-__global__ __launch_bounds__(kBwdThreads) void attn_bwd_dkv_bf16_kernel(AttnArgs a) {
+__device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg_id) {
     using TL = Tile<D>;
     constexpr int KK = D / 16;
     constexpr int DB = D / 32;
@@ -100,11 +100,11 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dkv_bf16_kernel(AttnArgs
     auto Ebuf = [&](int i) { return (MA_LDS float*)(aux + 2 * BM * 4) + i * BM; };
     auto Dbuf = [&](int i) { return (MA_LDS int64_t*)(aux + 4 * BM * 4) + i * BM; };
 
-    const int tid = threadIdx.x, lane = tid & 63;
+    const int tid = fresh_tid(), lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 31, hh = lane >> 5;
     int j, hk, b;
-    if (!map_work(blockIdx.x, a.B * a.T, a.T, a.Hkv, 1, a.map.kv_tile_order, j, hk, b)) return;
+    if (!map_work(wg_id, a.B * a.T, a.T, a.Hkv, 1, a.map.kv_tile_order, j, hk, b)) return;
     const int rbase = TL::row_base(lane), tbase = TL::tr_base(lane);
     const int G = a.Hq / a.Hkv;
     const int kw_lo = j * kTile + 32 * w, kw_hi = kw_lo + 31;
@@ -327,11 +327,26 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dkv_bf16_kernel(AttnArgs
     }
 }
 
+// One workgroup per work item, or -- with work queues in the tile map -- one per compute unit, pulling
+// items until none is left (see WorkQueue).
+template <int D, bool HAS_DOC>
+__global__ __launch_bounds__(kBwdThreads) void attn_bwd_dkv_bf16_kernel(AttnArgs a) {
+    extern __shared__ __align__(16) char smem_raw[];
+    MA_LDS int* box = (MA_LDS int*)((lds_ptr)smem_raw + (4 * Tile<D>::bytes(kStep) + 2 * kStep * (4 + 4 + 8)));
+    WorkQueue wq;
+    wq.init(a.map.work_counters, kQueueDkv, work_grid(a.B * a.T, a.Hkv, 1));
+    for (int id = wq.next(box); id >= 0; id = wq.next(box)) {
+        attn_bwd_dkv_bf16_item<D, HAS_DOC>(fresh_args(), id);
+        __syncthreads();  // the item's LDS (and the box) are free again
+    }
+    wq.leave();
+}
+
 // ------------------------------------------------------------------------------------------------
 // dQ
 // ------------------------------------------------------------------------------------------------
 template <int D, bool HAS_DOC>
-__global__ __launch_bounds__(kBwdThreads) void attn_bwd_dq_bf16_kernel(AttnArgs a) {
+__device__ __forceinline__ void attn_bwd_dq_bf16_item(KernArgs& a, const int wg_id) {
     using TL = Tile<D>;
     constexpr int KK = D / 16;
     constexpr int DB = D / 32;
@@ -343,11 +358,11 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dq_bf16_kernel(AttnArgs 
     auto Vbuf = [&](int i) { return lds0 + i * 2 * TL::bytes(BN) + TL::bytes(BN); };
     auto Dbuf = [&](int i) { return (MA_LDS int64_t*)(lds0 + 4 * TL::bytes(BN)) + i * BN; };
 
-    const int tid = threadIdx.x, lane = tid & 63;
+    const int tid = fresh_tid(), lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 31, hh = lane >> 5;
     int i, h, b;
-    if (!map_work(blockIdx.x, a.B * a.T, a.T, a.Hkv, a.Hq / a.Hkv, a.map.q_tile_order, i, h, b)) return;
+    if (!map_work(wg_id, a.B * a.T, a.T, a.Hkv, a.Hq / a.Hkv, a.map.q_tile_order, i, h, b)) return;
     const int rbase = TL::row_base(lane), tbase = TL::tr_base(lane);
     const int hk = h / (a.Hq / a.Hkv);
     const int qw_lo = i * kTile + 32 * w, qw_hi = qw_lo + 31;
@@ -570,6 +585,13 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_dq_bf16_kernel(AttnArgs 
     }
 }
 
+// One workgroup per work item.  (This kernel has many short items and no registers to spare: the
+// work queues that the forward and dK/dV kernels pull from cost it more than they gain.)
+template <int D, bool HAS_DOC>
+__global__ __launch_bounds__(kBwdThreads) void attn_bwd_dq_bf16_kernel(AttnArgs a) {
+    attn_bwd_dq_bf16_item<D, HAS_DOC>(fresh_args(), (int)blockIdx.x);
+}
+
 template <typename K>
 static int opt_in_lds(K kernel, size_t bytes, const char* name) {
     if (bytes <= 64 * 1024) return MA_OK;
@@ -599,10 +621,10 @@ static int bwd_dd(const AttnArgs& a, hipStream_t st) {
         if (rc) return rc;
     }
     if (a.stages & MA_BWD_DKV) {
-        const size_t lds_kv = (size_t)4 * Tile<D>::bytes(kStep) + 2 * kStep * (4 + 4 + 8);
+        const size_t lds_kv = (size_t)4 * Tile<D>::bytes(kStep) + 2 * kStep * (4 + 4 + 8) + 16;
         rc = opt_in_lds(attn_bwd_dkv_bf16_kernel<D, HAS_DOC>, lds_kv, "attn_bwd_dkv_bf16");
         if (rc) return rc;
-        hipLaunchKernelGGL((attn_bwd_dkv_bf16_kernel<D, HAS_DOC>), dim3(work_grid(a.B * a.T, a.Hkv, 1), 1, 1), dim3(kBwdThreads), lds_kv,
+        hipLaunchKernelGGL((attn_bwd_dkv_bf16_kernel<D, HAS_DOC>), dim3(queue_grid(work_grid(a.B * a.T, a.Hkv, 1), a.map.work_counters), 1, 1), dim3(kBwdThreads), lds_kv,
                            st, a);
         rc = check_launch("attn_bwd_dkv_bf16_kernel");
     }

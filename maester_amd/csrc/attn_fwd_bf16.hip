@@ -24,7 +24,7 @@ constexpr int kFwdBN = 64;  // kv rows per step
 constexpr int kPipe = 4;  // LDS fragment reads kept in flight ahead of the MFMAs
 
 template <int D, bool HAS_DOC>
-__global__ __launch_bounds__(kFwdThreads) void attn_fwd_bf16_kernel(AttnArgs a) {
+__device__ __forceinline__ void attn_fwd_bf16_item(KernArgs& a, const int wg_id) {
     using TL = Tile<D>;
     constexpr int KK = D / 16;  // contraction steps of S^T
     constexpr int DB = D / 32;  // 32-row blocks of O^T
@@ -36,11 +36,11 @@ __global__ __launch_bounds__(kFwdThreads) void attn_fwd_bf16_kernel(AttnArgs a) 
     auto Vbuf = [&](int i) { return lds0 + i * 2 * TL::bytes(BN) + TL::bytes(BN); };
     auto Dbuf = [&](int i) { return (MA_LDS int64_t*)(lds0 + 4 * TL::bytes(BN)) + i * BN; };
 
-    const int tid = threadIdx.x, lane = tid & 63;
+    const int tid = fresh_tid(), lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keep it in a scalar register
     const int r = lane & 31, hh = lane >> 5;
     int i, h, b;
-    if (!map_work(blockIdx.x, a.B * a.T, a.T, a.Hkv, a.Hq / a.Hkv, a.map.q_tile_order, i, h, b)) return;
+    if (!map_work(wg_id, a.B * a.T, a.T, a.Hkv, a.Hq / a.Hkv, a.map.q_tile_order, i, h, b)) return;
     const int hk = h / (a.Hq / a.Hkv);
     const int qw_lo = i * kTile + 32 * w, qw_hi = qw_lo + 31;
     const int q = qw_lo + r;
@@ -292,15 +292,30 @@ __global__ __launch_bounds__(kFwdThreads) void attn_fwd_bf16_kernel(AttnArgs a) 
     }
 }
 
+// One workgroup per work item, or -- with work queues in the tile map -- one per compute unit, pulling
+// items until none is left (see WorkQueue).
+template <int D, bool HAS_DOC>
+__global__ __launch_bounds__(kFwdThreads) void attn_fwd_bf16_kernel(AttnArgs a) {
+    extern __shared__ __align__(16) char smem_raw[];
+    MA_LDS int* box = (MA_LDS int*)((lds_ptr)smem_raw + (4 * Tile<D>::bytes(kFwdBN) + 2 * kFwdBN * 8));
+    WorkQueue wq;
+    wq.init(a.map.work_counters, kQueueFwd, work_grid(a.B * a.T, a.Hkv, a.Hq / a.Hkv));
+    for (int id = wq.next(box); id >= 0; id = wq.next(box)) {
+        attn_fwd_bf16_item<D, HAS_DOC>(fresh_args(), id);
+        __syncthreads();  // the item's LDS (and the box) are free again
+    }
+    wq.leave();
+}
+
 template <int D, bool HAS_DOC>
 static int fwd_dd(const AttnArgs& a, hipStream_t st) {
-    const size_t lds = (size_t)4 * Tile<D>::bytes(kFwdBN) + 2 * kFwdBN * 8;
+    const size_t lds = (size_t)4 * Tile<D>::bytes(kFwdBN) + 2 * kFwdBN * 8 + 16;  // K/V ring, kv ids, work-queue box
     if (lds > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_bf16_kernel<D, HAS_DOC>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return fail(MA_ERR_LAUNCH, "hipFuncSetAttribute(attn_fwd_bf16, %zu): %s", lds, hipGetErrorString(e));
     }
-    hipLaunchKernelGGL((attn_fwd_bf16_kernel<D, HAS_DOC>), dim3(work_grid(a.B * a.T, a.Hkv, a.Hq / a.Hkv), 1, 1), dim3(kFwdThreads), lds,
+    hipLaunchKernelGGL((attn_fwd_bf16_kernel<D, HAS_DOC>), dim3(queue_grid(work_grid(a.B * a.T, a.Hkv, a.Hq / a.Hkv), a.map.work_counters), 1, 1), dim3(kFwdThreads), lds,
                        st, a);
     return check_launch("attn_fwd_bf16_kernel");
 }

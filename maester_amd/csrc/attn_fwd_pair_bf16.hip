@@ -35,7 +35,7 @@ constexpr int kPairPipeK = MA_PAIR_PK;  // LDS fragment reads in flight ahead of
 constexpr int kPairPipeV = MA_PAIR_PV;
 
 template <int D, bool HAS_DOC>
-__global__ __launch_bounds__(kPairThreads) void attn_fwd_pair_bf16_kernel(AttnArgs a) {
+__device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int wg_id) {
     using TL = Tile<D>;
     constexpr int KK = D / 16;
     constexpr int DB = D / 32;
@@ -47,12 +47,12 @@ __global__ __launch_bounds__(kPairThreads) void attn_fwd_pair_bf16_kernel(AttnAr
     auto Vbuf = [&](int i) { return lds0 + i * 2 * TL::bytes(BN) + TL::bytes(BN); };
     auto Dbuf = [&](int i) { return (MA_LDS int64_t*)(lds0 + 4 * TL::bytes(BN)) + i * BN; };
 
-    const int tid = threadIdx.x, lane = tid & 63;
+    const int tid = fresh_tid(), lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 31, hh = lane >> 5;
     const int G = a.Hq / a.Hkv, GP = G / 2;  // head pairs per kv head
     int i, hp, b;
-    if (!map_work(blockIdx.x, a.B * a.T, a.T, a.Hkv, GP, a.map.q_tile_order, i, hp, b)) return;
+    if (!map_work(wg_id, a.B * a.T, a.T, a.Hkv, GP, a.map.q_tile_order, i, hp, b)) return;
     const int hk = hp / GP;
     const int h0 = hk * G + 2 * (hp % GP);   // the pair is (h0, h0 + 1)
     const int qw_lo = i * kTile + 32 * w, qw_hi = qw_lo + 31;
@@ -323,16 +323,31 @@ __global__ __launch_bounds__(kPairThreads) void attn_fwd_pair_bf16_kernel(AttnAr
     }
 }
 
+// One workgroup per work item, or -- with work queues in the tile map -- one per compute unit, pulling
+// items until none is left (see WorkQueue).
+template <int D, bool HAS_DOC>
+__global__ __launch_bounds__(kPairThreads) void attn_fwd_pair_bf16_kernel(AttnArgs a) {
+    extern __shared__ __align__(16) char smem_raw[];
+    MA_LDS int* box = (MA_LDS int*)((lds_ptr)smem_raw + (4 * Tile<D>::bytes(kPairBN) + 2 * kPairBN * 8 + 4));
+    WorkQueue wq;
+    wq.init(a.map.work_counters, kQueueFwd, work_grid(a.B * a.T, a.Hkv, a.Hq / a.Hkv / 2));
+    for (int id = wq.next(box); id >= 0; id = wq.next(box)) {
+        attn_fwd_pair_bf16_item<D, HAS_DOC>(fresh_args(), id);
+        __syncthreads();  // the item's LDS (and the box) are free again
+    }
+    wq.leave();
+}
+
 template <int D, bool HAS_DOC>
 static int pair_dd(const AttnArgs& a, hipStream_t st) {
-    const size_t lds = (size_t)4 * Tile<D>::bytes(kPairBN) + 2 * kPairBN * 8 + 16;  // K/V ring, kv ids, redo flag
+    const size_t lds = (size_t)4 * Tile<D>::bytes(kPairBN) + 2 * kPairBN * 8 + 16;  // K/V ring, kv ids, redo flag + work-queue box
     if (lds > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_pair_bf16_kernel<D, HAS_DOC>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return fail(MA_ERR_LAUNCH, "hipFuncSetAttribute(attn_fwd_pair_bf16, %zu): %s", lds, hipGetErrorString(e));
     }
     const int GP = a.Hq / a.Hkv / 2;
-    hipLaunchKernelGGL((attn_fwd_pair_bf16_kernel<D, HAS_DOC>), dim3(work_grid(a.B * a.T, a.Hkv, GP), 1, 1), dim3(kPairThreads), lds, st, a);
+    hipLaunchKernelGGL((attn_fwd_pair_bf16_kernel<D, HAS_DOC>), dim3(queue_grid(work_grid(a.B * a.T, a.Hkv, GP), a.map.work_counters), 1, 1), dim3(kPairThreads), lds, st, a);
     return check_launch("attn_fwd_pair_bf16_kernel");
 }
 

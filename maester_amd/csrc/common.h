@@ -56,6 +56,23 @@ struct AttnArgs {
     int stages;  // MA_BWD_* mask (backward only)
 };
 
+// The argument block as the per-item functions of the queue-driven kernels see it: in the constant
+// address space (scalar loads), behind a pointer the compiler cannot see through -- and the thread
+// id likewise.  Everything derived from either is then computed inside the item that uses it;
+// otherwise the compiler hoists all of it out of the loop over items and keeps it in registers
+// across the whole loop, which these kernels (512 registers per lane in use) cannot afford.
+typedef const __attribute__((address_space(4))) AttnArgs KernArgs;
+__device__ __forceinline__ KernArgs& fresh_args() {
+    KernArgs* p = (KernArgs*)__builtin_amdgcn_kernarg_segment_ptr();
+    asm volatile("" : "+s"(p));
+    return *p;
+}
+__device__ __forceinline__ int fresh_tid() {
+    int t = threadIdx.x;
+    asm volatile("" : "+v"(t));
+    return t;
+}
+
 int launch_attn_fwd_f32(const AttnArgs& a, hipStream_t st);
 int launch_attn_bwd_f32(const AttnArgs& a, hipStream_t st);
 int launch_attn_fwd_bf16(const AttnArgs& a, hipStream_t st);
@@ -102,6 +119,77 @@ __device__ __forceinline__ bool map_work(int id, int n_units, int T, int Hkv, in
     tile = __builtin_amdgcn_readfirstlane(u % T);
     head = __builtin_amdgcn_readfirstlane(hk * heads + g);
     return true;
+}
+
+// Where the ids handed to map_work come from.  Without counters (ma_tile_map.work_counters NULL) a
+// launch has one workgroup per id and each handles its blockIdx.  With counters a launch has one
+// workgroup per compute unit and the workgroups pull ids until none is left: id = 8 * k + x, with k
+// drawn from counter x -- first the counter of the workgroup's own XCD (blockIdx % 8, which keeps the
+// XCD affinity map_work builds into the ids), then, once that one is exhausted, the others'.  Pulling
+// keeps the longest-first order of the schedule but lets a compute unit start its next item the
+// moment it is done, instead of waiting for the hardware dispatcher's fixed round over the shader
+// engines.  The last workgroup to leave puts the counters back to zero for the next launch.
+//   counters: kWorkSlot ints per kernel kind (8 queues, then the count of workgroups that have left)
+#ifndef MA_LDS
+#define MA_LDS __attribute__((address_space(3)))
+#endif
+constexpr int kWorkSlot = 16;
+enum { kQueueFwd = 0, kQueueDq = 1, kQueueDkv = 2 };
+struct WorkQueue {
+    int32_t* ctr;   // nullptr: one id per workgroup
+    int per_xcd;    // ids per queue
+    bool first;
+    __device__ __forceinline__ void init(int32_t* counters, int kind, int total_ids) {
+        ctr = counters ? counters + kind * kWorkSlot : nullptr;
+        per_xcd = total_ids / kXcds;
+        first = true;
+    }
+    // The next id, or -1.  Every thread of the workgroup must call it; `box` is one int of LDS that
+    // nothing else uses, and a barrier must separate the return from the next call (the kernels
+    // end every item with one).
+    __device__ __forceinline__ int next(MA_LDS int* box) {
+        if (!ctr) {
+            const int id = first ? (int)blockIdx.x : -1;
+            first = false;
+            return id;
+        }
+        if (threadIdx.x == 0) {
+            const int x0 = blockIdx.x % kXcds;
+            int id = -1;
+            for (int t = 0; t < kXcds && id < 0; ++t) {
+                const int x = (x0 + t) % kXcds;
+                const int k = atomicAdd(ctr + x, 1);
+                if (k < per_xcd) id = k * kXcds + x;
+            }
+            *box = id;
+        }
+        __syncthreads();
+        return __builtin_amdgcn_readfirstlane(*box);
+    }
+    __device__ __forceinline__ void leave() {
+        if (ctr && threadIdx.x == 0) {
+            __threadfence();
+            if (atomicAdd(ctr + kXcds, 1) == (int)gridDim.x - 1)
+                for (int x = 0; x <= kXcds; ++x) atomicExch(ctr + x, 0);
+        }
+    }
+};
+// grid of a launch: one workgroup per id, or (with work queues) at most one per compute unit
+inline int compute_units() {
+    static int cached[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+    int c = cached[dev];
+    if (c <= 0) {
+        if (hipDeviceGetAttribute(&c, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || c <= 0) c = 256;
+        cached[dev] = c;
+    }
+    return c;
+}
+inline int queue_grid(int total_ids, const int32_t* counters) {
+    if (!counters) return total_ids;
+    const int cus = compute_units();
+    return total_ids < cus ? total_ids : cus;
 }
 
 // Walks `reps` times over the concatenation of two tile lists (partial tiles, then full tiles) of a

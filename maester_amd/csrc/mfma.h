@@ -32,7 +32,9 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef int64_t i64x2 __attribute__((ext_vector_type(2)));
 
+#ifndef MA_LDS
 #define MA_LDS __attribute__((address_space(3)))
+#endif
 typedef MA_LDS char* lds_ptr;
 
 // compile-time loop: f(std::integral_constant<int, I>{}) for I in [B, E)

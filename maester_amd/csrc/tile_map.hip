@@ -16,8 +16,10 @@ namespace ma {
 // (min, max) document id over the valid rows of every 128-row tile; one wave per tile.  Also clears
 // the counter of the hard-tile list.  With doc == nullptr only the counter is cleared.
 __global__ __launch_bounds__(256) void tile_ranges_kernel(const int64_t* __restrict__ doc, int B, int S, int T,
-                                                          int64_t* __restrict__ rng, int* __restrict__ n_hard) {
+                                                          int64_t* __restrict__ rng, int* __restrict__ n_hard,
+                                                          int32_t* __restrict__ work_counters) {
     if (blockIdx.x == 0 && threadIdx.x == 0) *n_hard = 0;
+    if (blockIdx.x == 0 && work_counters && threadIdx.x < MA_WORK_COUNTERS) work_counters[threadIdx.x] = 0;
     const int tile = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
     if (!doc || tile >= B * T) return;
     const int b = tile / T, r0 = (tile % T) * kTile;
@@ -203,7 +205,8 @@ int launch_tile_map(const int64_t* doc, int B, int S, int causal, int64_t window
     int64_t* rng = (int64_t*)((char*)ws + ((ntiles + 15) & ~(size_t)15));
     int* n_hard = (int*)(rng + (size_t)B * T * 2);
     int32_t* hard = (int32_t*)((char*)n_hard + 16);
-    hipLaunchKernelGGL(tile_ranges_kernel, dim3((B * T + 3) / 4), dim3(256), 0, st, doc, B, S, T, rng, n_hard);
+    hipLaunchKernelGGL(tile_ranges_kernel, dim3((B * T + 3) / 4), dim3(256), 0, st, doc, B, S, T, rng, n_hard,
+                       out.work_counters);
     int rc = check_launch("tile_ranges_kernel");
     if (rc) return rc;
     hipLaunchKernelGGL(classify_easy_kernel, dim3((unsigned)((ntiles + 255) / 256)), dim3(256), 0, st, rng, doc ? 1 : 0, B, S, T,

@@ -38,6 +38,9 @@ class TileMap:
     kv_tile_order: torch.Tensor | None = None
     # (min, max) document id of every 32-row block, int64 [B, 2*ceil(S/64), 2]; None without document ids
     block_doc_range: torch.Tensor | None = None
+    # work queues of the attention kernels, int32 [64], zeroed by the build (launches that share a
+    # tile map must be stream-ordered); None = one workgroup per work item
+    work_counters: torch.Tensor | None = None
 
     NAMES = ("kv_num_blocks", "kv_indices", "full_kv_num_blocks", "full_kv_indices",
              "q_num_blocks", "q_indices", "full_q_num_blocks", "full_q_indices")
@@ -47,7 +50,8 @@ class TileMap:
 
     def c_struct(self) -> _lib.MaTileMap:
         ptrs = [c_void_p(getattr(self, n).data_ptr()) for n in self.NAMES]
-        ptrs += [None if t is None else c_void_p(t.data_ptr()) for t in (self.q_tile_order, self.kv_tile_order, self.block_doc_range)]
+        ptrs += [None if t is None else c_void_p(t.data_ptr()) for t in (self.q_tile_order, self.kv_tile_order, self.block_doc_range,
+                                                                           self.work_counters)]
         return _lib.MaTileMap(*ptrs)
 
     @property
@@ -82,7 +86,8 @@ def build_tile_map(document_ids: torch.Tensor | None, batch_size: int, seq_len: 
     order = torch.empty(2, batch_size * T, dtype=torch.int32, device=device)
     tm = TileMap(nums[0], idxs[0], nums[1], idxs[1], nums[2], idxs[2], nums[3], idxs[3],
                  seq_len=seq_len, causal=bool(causal), window=sliding_window, q_tile_order=order[0],
-                 kv_tile_order=order[1])
+                 kv_tile_order=order[1],
+                 work_counters=torch.empty(_lib.MA_WORK_COUNTERS, dtype=torch.int32, device=device))
     if document_ids is not None:
         nblk = 2 * ((seq_len + 63) // 64)   # two 32-row blocks per 64-row step, the last step padded
         tm.block_doc_range = torch.empty(batch_size, nblk, 2, dtype=torch.int64, device=device)

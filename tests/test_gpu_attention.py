@@ -221,6 +221,29 @@ def test_full_size_backward_slices(gpu, name):
         torch.cuda.empty_cache()
 
 
+@pytest.mark.parametrize("heads", [(4, 2), (3, 3)], ids=["pair", "single"])
+def test_work_queues_give_the_same_results_and_reset_themselves(gpu, heads):
+    """With work counters in the tile map the forward and dK/dV kernels run one workgroup per compute
+    unit that pulls work items; without, one workgroup per item.  Same bits either way, and the
+    counters are back at zero after every launch (so launches can follow one another)."""
+    Hq, Hkv = heads
+    B, S, D = 3, 1500, 128
+    q, k, v, do = (t.to(gpu) for t in _qkv(B, S, Hq, Hkv, D, torch.bfloat16, 11))
+    ids = _ids(B, S, 12, "docs").to(gpu)
+    tm = build_tile_map(ids, B, S, True, None)
+    assert tm.work_counters is not None and int(tm.work_counters.abs().sum()) == 0
+    results = []
+    for counters in (tm.work_counters, None, tm.work_counters):
+        tm.work_counters = counters
+        out, lse = attention_forward(q, k, v, tm, ids, D ** -0.5, True, None)
+        grads = attention_backward(q, k, v, out, do, lse, tm, ids, D ** -0.5, True, None)
+        results.append((out, lse) + tuple(grads))
+        if counters is not None:
+            assert int(counters.abs().sum()) == 0
+    for other in results[1:]:
+        assert all(torch.equal(x, y) for x, y in zip(results[0], other))
+
+
 @pytest.mark.parametrize("heads", [(2, 1), (4, 2), (2, 2)], ids=["pair_g2", "pair_g2_hkv2", "single_g1"])
 @pytest.mark.parametrize("D", [128, 256])
 def test_bf16_forward_scores_that_outgrow_the_first_block(gpu, heads, D):

@@ -156,3 +156,16 @@ def test_gemma_module_mirrors_reference_interface():
     with pytest.raises(NotImplementedError):
         attn.set_backend("flex")
     attn.set_backend("hip")
+
+
+def test_tile_map_struct_matches_the_header():
+    """The ctypes mirror of ma_tile_map has the header's fields, in the header's order."""
+    import os
+    import re
+    hdr = open(os.path.join(os.path.dirname(__file__), "..", "include", "maester_attn.h")).read()
+    body = hdr[hdr.index("typedef struct ma_tile_map {"):hdr.index("} ma_tile_map;")]
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    fields = re.findall(r"\b(?:int32_t|int64_t)\s*\*\s*(\w+)\s*;", body)
+    assert fields == [n for n, _ in MaTileMap._fields_] and len(fields) == 12
+    assert int(re.search(r"#define MA_WORK_COUNTERS (\d+)", hdr).group(1)) == _lib.MA_WORK_COUNTERS
+    assert int(re.search(r"#define MA_DOC_BLOCK (\d+)", hdr).group(1)) == _lib.MA_DOC_BLOCK
