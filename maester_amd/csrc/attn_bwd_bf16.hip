@@ -149,23 +149,26 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
     // q steps of the kv tile, for each of the G query heads in turn, from the last q tile down (see
     // ListWalk); limits inside which a 32-row q block of a partial tile can be visible to this wave
     const bool windowed = a.window >= 0;
-    StepWalk<BM> st;
-    {
-        int lo, hi;
-        visibility_limits(true, j * kTile, j * kTile + kTile - 1, BM, bounded, wlim, windowed, lo, hi);
-        int n_partial, n_full;
-        scalar_load2(a.map.q_num_blocks + mrow, a.map.full_q_num_blocks + mrow, n_partial, n_full);
-        st.init(a.map.q_indices + mrow * a.T, n_partial, a.map.full_q_indices + mrow * a.T, n_full, G, true, a.S, lo, hi);
-    }
     int blk_lo, blk_hi;
     visibility_limits(true, kw_lo, kw_hi, 32, bounded, wlim, windowed, blk_lo, blk_hi);
-    // document-id ranges: of the wave's own kv rows now, of the two q blocks of a step at each step
+    // document-id range of the wave's own kv rows (the step table tests the q blocks against it)
     const bool use_rng = HAS_DOC && a.map.block_doc_range != nullptr;
     const int64_t* rng_row = use_rng ? a.map.block_doc_range + (size_t)b * (2 * ((a.S + 63) / 64)) * 2 : nullptr;
     DocRange own;
     if (use_rng) {
         own.load(rng_row + (size_t)(min(kw_lo, a.S - 1) / MA_DOC_BLOCK) * 2);
         own.ready();
+    }
+    StepTable<BM> st;
+    {
+        int lo, hi;
+        visibility_limits(true, j * kTile, j * kTile + kTile - 1, BM, bounded, wlim, windowed, lo, hi);
+        int n_partial, n_full;
+        scalar_load2(a.map.q_num_blocks + mrow, a.map.full_q_num_blocks + mrow, n_partial, n_full);
+        st.init(a.map.q_indices + mrow * a.T, n_partial, a.map.full_q_indices + mrow * a.T, n_full, G, true, a.S, lo, hi,
+                blk_lo, blk_hi, rng_row, use_rng ? own.lo() : 0, use_rng ? own.hi() : 0,
+                (MA_LDS uint32_t*)(aux + 2 * BM * (4 + 4 + 8) + 16) + w * 64);
+        st.prime();
     }
 
     DirectStager<D, BM, NW> sq;  // the Q and dO tiles have the same shape: one set of slots
@@ -178,13 +181,13 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
     // global sources of the step the iterator stands on
     const char *qsrc = nullptr, *gsrc = nullptr;
     auto locate = [&]() {
-        const int h = hk * G + st.walk.rep;
+        const int h = hk * G + st.rep;
         qsrc = qhead + (uint64_t)(uint32_t)h * (uint32_t)(a.q.stride_h * 2) + (uint64_t)(uint32_t)st.r0 * qsb;
         gsrc = ghead + (uint64_t)(uint32_t)h * (uint32_t)(a.dout.stride_h * 2) + (uint64_t)(uint32_t)st.r0 * gsb;
     };
     auto issue_rows = [&]() {  // per-row lse / delta / document id of that step
         if (tid < BM) {
-            const int h = hk * G + st.walk.rep;
+            const int h = hk * G + st.rep;
             const int qq = min(st.r0 + tid, a.S - 1);
             const size_t row = ((size_t)b * a.Hq + h) * a.S + qq;
             lse_next = a.lse[row];  // converted to log2 units when it is written to LDS
@@ -195,9 +198,9 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
     auto issue_q = [&](int buf) { sq.issue((const __bf16*)qsrc, Qbuf(buf), w, lane, min(BM, a.S - st.r0), a.q.stride_s); };
     auto issue_g = [&](int buf) { sq.issue((const __bf16*)gsrc, Gbuf(buf), w, lane, min(BM, a.S - st.r0), a.dout.stride_s); };
     const int my_runs = decltype(sq)::runs_of(w);
-    bool have = st.first();
+    bool have = st.next();
     int q0 = st.r0;
-    bool partial = st.partial;
+    bool partial = st.partial, act0 = st.act0, act1 = st.act1;
     if (have) {
         locate();
         issue_q(0);
@@ -211,8 +214,6 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
         MA_LDS float* lse2s = Lbuf(cur);
         MA_LDS float* dls = Ebuf(cur);
         MA_LDS int64_t* qdoc = Dbuf(cur);
-        DocRange2 rng;
-        if (use_rng && partial) rng.load(rng_row + (size_t)(q0 / MA_DOC_BLOCK) * 2);
         if (tid < BM) {
             lse2s[tid] = lse_next * kLog2e;
             dls[tid] = dl_next;
@@ -223,23 +224,18 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
 
         const int cq0 = q0;
         const bool cpartial = partial;
+        const bool skip[BM / 32] = {!act0, !act1};  // blocks in which this wave has nothing to do
         have = st.next();
         // The tile loads of the next step are spread over this step's first MFMA chains, one run
         // every few MFMAs (Q tile in the first 32-row block, dO tile in the second): issued in one
         // burst they fill the memory pipeline and stall the wave with the matrix cores idle.  A
         // ragged last tile, or a block that is skipped, issues its tile at once.
-        bool skip[BM / 32];
-#pragma unroll
-        for (int mb = 0; mb < BM / 32; ++mb) skip[mb] = !block_visible(cq0 + 32 * mb, a.S, cpartial, blk_lo, blk_hi);
-        if (use_rng && cpartial) {  // no q row of the block shares a document with the wave's kv rows
-            rng.ready();
-#pragma unroll
-            for (int mb = 0; mb < BM / 32; ++mb) skip[mb] |= !rng.meets(mb, own.lo(), own.hi());
-        }
         int pace = 0;
         if (have) {
             q0 = st.r0;
             partial = st.partial;
+            act0 = st.act0;
+            act1 = st.act1;
             locate();
             issue_rows();
             const bool spread = (q0 + BM <= a.S) & !skip[0] & !skip[1];
@@ -390,19 +386,27 @@ __device__ __forceinline__ void attn_bwd_dq_bf16_item(KernArgs& a, const int wg_
     // below in the memory pipeline, and the first K/V tiles can be requested as soon as they return.
     const size_t mrow = (size_t)b * a.T + i;
     const bool windowed = a.window >= 0;
-    StepWalk<BN> st;
+    int blk_lo, blk_hi;
+    visibility_limits(false, qw_lo, qw_hi, 32, bounded, wlim, windowed, blk_lo, blk_hi);
+    // document-id range of the wave's own q rows (the step table tests the kv blocks against it)
+    const bool use_rng = HAS_DOC && a.map.block_doc_range != nullptr;
+    const int64_t* rng_row = use_rng ? a.map.block_doc_range + (size_t)b * (2 * ((a.S + 63) / 64)) * 2 : nullptr;
+    DocRange own;
+    if (use_rng) {  // (load and wait stay adjacent: the registers of a scalar load in flight must not be touched)
+        own.load(rng_row + (size_t)(min(qw_lo, a.S - 1) / MA_DOC_BLOCK) * 2);
+        own.ready();
+    }
+    StepTable<BN> st;
     {
         int lo, hi;
         visibility_limits(false, i * kTile, i * kTile + kTile - 1, BN, bounded, wlim, windowed, lo, hi);
         int n_partial, n_full;
         scalar_load2(a.map.kv_num_blocks + mrow, a.map.full_kv_num_blocks + mrow, n_partial, n_full);
-        st.init(a.map.kv_indices + mrow * a.T, n_partial, a.map.full_kv_indices + mrow * a.T, n_full, 1, false, a.S, lo, hi);
+        st.init(a.map.kv_indices + mrow * a.T, n_partial, a.map.full_kv_indices + mrow * a.T, n_full, 1, false, a.S, lo, hi,
+                blk_lo, blk_hi, rng_row, use_rng ? own.lo() : 0, use_rng ? own.hi() : 0,
+                (MA_LDS uint32_t*)(lds0 + 4 * TL::bytes(BN) + 2 * BN * 8 + 16) + w * 64);
+        st.prime();
     }
-    int blk_lo, blk_hi;
-    visibility_limits(false, qw_lo, qw_hi, 32, bounded, wlim, windowed, blk_lo, blk_hi);
-    // document-id ranges: of the wave's own q rows now, of the two kv blocks of a step at each step
-    const bool use_rng = HAS_DOC && a.map.block_doc_range != nullptr;
-    const int64_t* rng_row = use_rng ? a.map.block_doc_range + (size_t)b * (2 * ((a.S + 63) / 64)) * 2 : nullptr;
 
     // Q and dO rows of the wave go straight from global memory into MFMA operand fragments: lane
     // (r, hh) holds elements 16*kk + 8*hh .. +7 of row qw_lo + r, one 16-byte load each (the two
@@ -423,13 +427,6 @@ __device__ __forceinline__ void attn_bwd_dq_bf16_item(KernArgs& a, const int wg_
 #pragma unroll
             for (int kk = 0; kk < KK; ++kk) of[kk] = *(const u32x4*)(orow + 16 * kk);
         }
-    }
-
-    // (load and wait stay adjacent: the registers of a scalar load in flight must not be touched)
-    DocRange own;
-    if (use_rng) {
-        own.load(rng_row + (size_t)(min(qw_lo, a.S - 1) / MA_DOC_BLOCK) * 2);
-        own.ready();
     }
 
     f32x16 acc[DB];
@@ -453,9 +450,9 @@ __device__ __forceinline__ void attn_bwd_dq_bf16_item(KernArgs& a, const int wg_
         if (HAS_DOC && st.partial && tid < BN) kd_next = drow[min(st.r0 + tid, a.S - 1)];
     };
     const int my_runs = decltype(sk)::runs_of(w);
-    bool have = st.first();
+    bool have = st.next();
     int k0 = st.r0;
-    bool partial = st.partial;
+    bool partial = st.partial, act0 = st.act0, act1 = st.act1;
     if (have) {
         issue_k(0);
         issue_v(0);
@@ -486,23 +483,14 @@ __device__ __forceinline__ void attn_bwd_dq_bf16_item(KernArgs& a, const int wg_
         const int cur = n & 1;
         const lds_ptr Ks = Kbuf(cur), Vs = Vbuf(cur);
         MA_LDS int64_t* kdoc = Dbuf(cur);
-        DocRange2 rng;
-        if (use_rng && partial) rng.load(rng_row + (size_t)(k0 / MA_DOC_BLOCK) * 2);
         if (HAS_DOC && partial && tid < BN) kdoc[tid] = kd_next;
         wait_vmem();
         __syncthreads();
 
         const int ck0 = k0;
         const bool cpartial = partial;
+        const bool skip[BN / 32] = {!act0, !act1};  // blocks in which this wave has nothing to do
         have = st.next();
-        bool skip[BN / 32];
-#pragma unroll
-        for (int nb = 0; nb < BN / 32; ++nb) skip[nb] = !block_visible(ck0 + 32 * nb, a.S, cpartial, blk_lo, blk_hi);
-        if (use_rng && cpartial) {  // no kv row of the block shares a document with the wave's q rows
-            rng.ready();
-#pragma unroll
-            for (int nb = 0; nb < BN / 32; ++nb) skip[nb] |= !rng.meets(nb, own.lo(), own.hi());
-        }
         // The tile loads of the next step are spread over this step's first MFMA chains (K tile in
         // the first 32-row block, V tile in the second), see the dK/dV kernel.
         int pace = 0;
@@ -510,6 +498,8 @@ __device__ __forceinline__ void attn_bwd_dq_bf16_item(KernArgs& a, const int wg_
         if (have) {
             k0 = st.r0;
             partial = st.partial;
+            act0 = st.act0;
+            act1 = st.act1;
             ksrc = (const __bf16*)((const char*)kp + (uint64_t)(uint32_t)k0 * ksb);
             vsrc = (const __bf16*)((const char*)vp + (uint64_t)(uint32_t)k0 * vsb);
             issue_ids();
@@ -612,7 +602,7 @@ static int bwd_dd(const AttnArgs& a, hipStream_t st) {
         if (rc) return rc;
     }
     if (a.stages & MA_BWD_DQ) {  // first: the dK/dV kernel reads the delta this one may be writing
-        const size_t lds_q = (size_t)4 * Tile<D>::bytes(kStep) + 2 * kStep * 8;  // K/V ring, kv document ids
+        const size_t lds_q = (size_t)4 * Tile<D>::bytes(kStep) + 2 * kStep * 8 + 16 + (kBwdThreads / 64) * 256;  // K/V ring, kv document ids, step tables
         rc = opt_in_lds(attn_bwd_dq_bf16_kernel<D, HAS_DOC>, lds_q, "attn_bwd_dq_bf16");
         if (rc) return rc;
         hipLaunchKernelGGL((attn_bwd_dq_bf16_kernel<D, HAS_DOC>), dim3(work_grid(a.B * a.T, a.Hkv, a.Hq / a.Hkv), 1, 1), dim3(kBwdThreads),
@@ -621,7 +611,7 @@ static int bwd_dd(const AttnArgs& a, hipStream_t st) {
         if (rc) return rc;
     }
     if (a.stages & MA_BWD_DKV) {
-        const size_t lds_kv = (size_t)4 * Tile<D>::bytes(kStep) + 2 * kStep * (4 + 4 + 8) + 16;
+        const size_t lds_kv = (size_t)4 * Tile<D>::bytes(kStep) + 2 * kStep * (4 + 4 + 8) + 16 + (kBwdThreads / 64) * 256;  // + work-queue box, step tables
         rc = opt_in_lds(attn_bwd_dkv_bf16_kernel<D, HAS_DOC>, lds_kv, "attn_bwd_dkv_bf16");
         if (rc) return rc;
         hipLaunchKernelGGL((attn_bwd_dkv_bf16_kernel<D, HAS_DOC>), dim3(queue_grid(work_grid(a.B * a.T, a.Hkv, 1), a.map.work_counters), 1, 1), dim3(kBwdThreads), lds_kv,

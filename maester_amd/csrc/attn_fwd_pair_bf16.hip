@@ -74,7 +74,7 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
     const float sl2 = a.scale * kLog2e;
 
     const size_t mrow = (size_t)b * a.T + i;
-    StepWalk<BN> st;
+    StepTable<BN> st;
     int blk_lo, blk_hi;
     visibility_limits(false, qw_lo, qw_hi, 32, bounded, wlim, windowed, blk_lo, blk_hi);
     const bool use_rng = HAS_DOC && a.map.block_doc_range != nullptr;
@@ -96,18 +96,23 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
     // index loads are back, the first K/V tiles -- all in flight together.
     bool have;
     int k0;
-    bool partial;
+    bool partial, act0, act1;  // of the step the walk stands on: tile kind, blocks this wave has work in
+    MA_LDS uint32_t* steps_slot = (MA_LDS uint32_t*)(lds0 + 4 * TL::bytes(BN) + 2 * BN * 8 + 16) + w * 64;
     auto walk_init = [&]() {
         int lo, hi;
         visibility_limits(false, i * kTile, i * kTile + kTile - 1, BN, bounded, wlim, windowed, lo, hi);
         int n_partial, n_full;
         scalar_load2(a.map.kv_num_blocks + mrow, a.map.full_kv_num_blocks + mrow, n_partial, n_full);
-        st.init(a.map.kv_indices + mrow * a.T, n_partial, a.map.full_kv_indices + mrow * a.T, n_full, 1, false, a.S, lo, hi);
+        st.init(a.map.kv_indices + mrow * a.T, n_partial, a.map.full_kv_indices + mrow * a.T, n_full, 1, false, a.S, lo, hi,
+                blk_lo, blk_hi, use_rng ? rng_row : nullptr, use_rng ? own.lo() : 0, use_rng ? own.hi() : 0, steps_slot);
+        st.prime();
     };
     auto walk_first = [&]() {
-        have = st.first();
+        have = st.next();
         k0 = st.r0;
         partial = st.partial;
+        act0 = st.act0;
+        act1 = st.act1;
         if (have) {
             const int rows_valid = min(BN, a.S - k0);
             sk.issue((const __bf16*)(kp + (uint64_t)(uint32_t)k0 * ksb), Kbuf(0), w, lane, rows_valid, a.k.stride_s);
@@ -152,23 +157,14 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
         const int cur = n & 1;
         const lds_ptr Ks = Kbuf(cur), Vs = Vbuf(cur);
         MA_LDS int64_t* kdoc = Dbuf(cur);
-        DocRange2 rng;
-        if (use_rng && partial) rng.load(rng_row + (size_t)(k0 / MA_DOC_BLOCK) * 2);
         if (HAS_DOC && partial && tid < BN) kdoc[tid] = kd_next;
         wait_vmem();
         __syncthreads();
 
         const int ck0 = k0;
         const bool cpartial = partial;
+        const bool act[2] = {act0, act1};
         have = st.next();
-        bool act[2];
-#pragma unroll
-        for (int nb = 0; nb < 2; ++nb) act[nb] = block_visible(ck0 + 32 * nb, a.S, cpartial, blk_lo, blk_hi);
-        if (use_rng && cpartial) {
-            rng.ready();
-#pragma unroll
-            for (int nb = 0; nb < 2; ++nb) act[nb] &= rng.meets(nb, own.lo(), own.hi());
-        }
         // the tile loads of the next step ride in the chains of the first active block (K in its S^T
         // chain, V in its O^T chain); a ragged last tile or a step without chains issues them at once
         int pace = 0;
@@ -177,6 +173,8 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
         if (have) {
             k0 = st.r0;
             partial = st.partial;
+            act0 = st.act0;
+            act1 = st.act1;
             ksrc = kp + (uint64_t)(uint32_t)k0 * ksb;
             vsrc = vp + (uint64_t)(uint32_t)k0 * vsb;
             if (HAS_DOC && partial && tid < BN) kd_next = drow[min(k0 + tid, a.S - 1)];
@@ -340,7 +338,7 @@ __global__ __launch_bounds__(kPairThreads) void attn_fwd_pair_bf16_kernel(AttnAr
 
 template <int D, bool HAS_DOC>
 static int pair_dd(const AttnArgs& a, hipStream_t st) {
-    const size_t lds = (size_t)4 * Tile<D>::bytes(kPairBN) + 2 * kPairBN * 8 + 16;  // K/V ring, kv ids, redo flag + work-queue box
+    const size_t lds = (size_t)4 * Tile<D>::bytes(kPairBN) + 2 * kPairBN * 8 + 16 + (kPairThreads / 64) * 256;  // K/V ring, kv ids, redo flag + work-queue box, step tables
     if (lds > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_pair_bf16_kernel<D, HAS_DOC>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);

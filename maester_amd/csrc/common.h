@@ -292,6 +292,99 @@ struct StepWalk {
         }
     }
 };
+// The same walk, resolved ahead of time.  Per step the walk above costs a wave some hundred scalar
+// and branch instructions (list bookkeeping, visibility tests, the id-range test of both 32-row
+// blocks with its scalar loads), and a wave that has its SIMD to itself pays the full latency of
+// every one of them between two MFMA chains.  Here a wave works the steps out 64 at a time, one
+// candidate step per lane, and keeps them as one word per step in its own slice of LDS:
+//     bits 0..23 first row of the step, 24..28 pass over the lists (the query head of the dK/dV
+//     kernel), 29 / 30 the wave has something to do in the second / first 32-row block, 31 partial tile
+// so that handing out a step is one LDS word (read a step ahead), a few bit operations and a
+// compare.  Every wave of a workgroup derives the same sequence of steps (same inputs); only the
+// two block bits are its own.  Filling takes a few vector loads and is needed once per 64 candidates.
+template <int STEP>
+struct StepTable {
+    static_assert(kTile % STEP == 0 && STEP == 64, "two 32-row blocks per step");
+    static constexpr int kPerTile = kTile / STEP;
+    const int32_t *pl, *fl;        // partial / full tile lists of the row
+    int np, n, reps;
+    bool backward;
+    int S, vis_lo, vis_hi;         // visibility of a step of a partial tile (the workgroup's rows)
+    int blk_lo, blk_hi;            // ... of one of its 32-row blocks (the wave's rows)
+    const int64_t* rng;            // (min, max) document id per 32-row block of the batch row, or nullptr
+    int64_t own_lo, own_hi;        // id range of the wave's own rows
+    MA_LDS uint32_t* slot;         // 64 words of LDS of this wave
+    int total, cbase, cnt, pos;
+    uint32_t ahead;                // the entry after the current one (per lane copy of an LDS word)
+
+    __device__ __forceinline__ void init(const int32_t* partial_list, int n_partial, const int32_t* full_list, int n_full,
+                                         int repeats, bool reverse, int seq_len, int lo, int hi, int wave_lo, int wave_hi,
+                                         const int64_t* block_ranges, int64_t own_min, int64_t own_max, MA_LDS uint32_t* lds_slot) {
+        pl = partial_list; fl = full_list; np = n_partial; n = n_partial + n_full; reps = repeats; backward = reverse;
+        S = seq_len; vis_lo = lo; vis_hi = hi; blk_lo = wave_lo; blk_hi = wave_hi;
+        rng = block_ranges; own_lo = own_min; own_hi = own_max; slot = lds_slot;
+        total = n * kPerTile * repeats; cbase = 0; cnt = 0; pos = 0; ahead = 0;
+        r0 = 0; rep = 0; partial = act0 = act1 = false;
+    }
+    // works out candidates cbase .. cbase + 63 and keeps the visible ones; returns how many
+    __device__ __forceinline__ int fill() {
+        const int lane = __lane_id();
+        const int c = cbase + lane;
+        const bool valid = c < total;
+        const int per_pass = n * kPerTile;
+        const int cc = valid ? c : 0;
+        const int rep = cc / per_pass, wi = cc - rep * per_pass;
+        const int it = wi / kPerTile, half = wi - it * kPerTile;
+        const int idx = backward ? n - 1 - it : it;
+        const bool partial = idx < np;
+        int tile = 0;
+        if (valid) tile = partial ? pl[idx] : fl[idx - np];
+        const int r0 = tile * kTile + half * STEP;
+        const bool vis = valid & (r0 < S) & (!partial | ((r0 >= vis_lo) & (r0 <= vis_hi)));
+        bool act0 = block_inside(r0, partial), act1 = block_inside(r0 + 32, partial);
+        if (rng && partial && vis) {  // no row of the block shares a document with the wave's own rows
+            const int64_t* e = rng + (size_t)(r0 / 32) * 2;
+            act0 &= (e[0] <= own_hi) & (e[1] >= own_lo);
+            act1 &= (e[2] <= own_hi) & (e[3] >= own_lo);
+        }
+        const uint32_t word = (uint32_t)r0 | ((uint32_t)rep << 24) | ((uint32_t)act1 << 29) | ((uint32_t)act0 << 30) | ((uint32_t)partial << 31);
+        const uint64_t mask = __ballot(vis);
+        const int at = __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0));
+        if (vis) slot[at] = word;
+        cbase += 64;
+        return __builtin_popcountll(mask);
+    }
+    __device__ __forceinline__ bool block_inside(int r0, bool partial) const {
+        return (r0 < S) & (!partial | ((r0 >= blk_lo) & (r0 <= blk_hi)));
+    }
+    // the next 64 candidates that hold a step at all; false when the walk is over.  prime() right
+    // after init(): the loads of the first fill are then ahead of whatever the kernel requests next.
+    __device__ __forceinline__ bool refill() {
+        cnt = 0;
+        while (cnt == 0 && cbase < total) cnt = fill();
+        pos = 0;
+        ahead = slot[0];
+        return cnt != 0;
+    }
+    __device__ __forceinline__ void prime() { refill(); }
+    // Moves on to the next step (false when the walk is over): its first row, the pass over the
+    // lists it belongs to, the kind of its tile, and whether this wave has work in its two blocks.
+    int r0, rep;
+    bool partial, act0, act1;
+    __device__ __forceinline__ bool next() {
+        if (pos == cnt && !refill()) return false;
+        const uint32_t word = __builtin_amdgcn_readfirstlane(ahead);
+        ++pos;
+        ahead = slot[pos & 63];  // read now, used at the next call
+        r0 = (int)(word & 0xffffffu);
+        rep = (int)((word >> 24) & 31u);
+        act1 = (word >> 29) & 1u;
+        act0 = (word >> 30) & 1u;
+        partial = (word >> 31) != 0;
+        return true;
+    }
+};
+
 // the same test for a block of rows starting at r0 (bounds of the wave's own rows)
 __device__ __forceinline__ bool block_visible(int r0, int S, bool partial, int lo, int hi) {
     return (r0 < S) & (!partial | ((r0 >= lo) & (r0 <= hi)));
