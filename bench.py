@@ -221,7 +221,7 @@ def main():
     base = sp.D * sp.Hq * wl.n_pairs
     kern = {
         # query heads that share a kv head go through the pair kernel when they come in pairs
-        ("attn_fwd_pair_bf16_kernel" if (sp.Hq // sp.Hkv) % 2 == 0 and sp.dtype == torch.bfloat16 else "attn_fwd_bf16_kernel"):
+        ("attn_fwd_pair_bf16_kernel" if (sp.Hq // sp.Hkv) % 2 == 0 and sp.D >= 256 and sp.dtype == torch.bfloat16 else "attn_fwd_bf16_kernel"):
             {"ms": t_fwd, "algorithmic_flops": 4 * base},
         "attn_bwd_dkv_bf16_kernel": {"ms": t_dkv, "algorithmic_flops": 6 * base},   # dP, dV, dK
         "attn_bwd_dq_bf16_kernel": {"ms": t_dq, "algorithmic_flops": 2 * base},     # dQ

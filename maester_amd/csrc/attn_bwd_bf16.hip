@@ -19,6 +19,10 @@
 #include "common.h"
 #include "mfma.h"
 
+#ifndef MA_DKV_WAVES
+#define MA_DKV_WAVES 1
+#endif
+
 namespace ma {
 
 constexpr int kBwdThreads = 256;
@@ -326,7 +330,7 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
 // One workgroup per work item, or -- with work queues in the tile map -- one per compute unit, pulling
 // items until none is left (see WorkQueue).
 template <int D, bool HAS_DOC>
-__global__ __launch_bounds__(kBwdThreads) void attn_bwd_dkv_bf16_kernel(AttnArgs a) {
+__global__ __launch_bounds__(kBwdThreads, D <= 128 ? MA_DKV_WAVES : 1) void attn_bwd_dkv_bf16_kernel(AttnArgs a) {
     extern __shared__ __align__(16) char smem_raw[];
     MA_LDS int* box = (MA_LDS int*)((lds_ptr)smem_raw + (4 * Tile<D>::bytes(kStep) + 2 * kStep * (4 + 4 + 8)));
     WorkQueue wq;
@@ -578,7 +582,7 @@ __device__ __forceinline__ void attn_bwd_dq_bf16_item(KernArgs& a, const int wg_
 // One workgroup per work item.  (This kernel has many short items and no registers to spare: the
 // work queues that the forward and dK/dV kernels pull from cost it more than they gain.)
 template <int D, bool HAS_DOC>
-__global__ __launch_bounds__(kBwdThreads) void attn_bwd_dq_bf16_kernel(AttnArgs a) {
+__global__ __launch_bounds__(kBwdThreads, D <= 128 ? 2 : 1) void attn_bwd_dq_bf16_kernel(AttnArgs a) {
     attn_bwd_dq_bf16_item<D, HAS_DOC>(fresh_args(), (int)blockIdx.x);
 }
 
@@ -614,7 +618,8 @@ static int bwd_dd(const AttnArgs& a, hipStream_t st) {
         const size_t lds_kv = (size_t)4 * Tile<D>::bytes(kStep) + 2 * kStep * (4 + 4 + 8) + 16 + (kBwdThreads / 64) * 256;  // + work-queue box, step tables
         rc = opt_in_lds(attn_bwd_dkv_bf16_kernel<D, HAS_DOC>, lds_kv, "attn_bwd_dkv_bf16");
         if (rc) return rc;
-        hipLaunchKernelGGL((attn_bwd_dkv_bf16_kernel<D, HAS_DOC>), dim3(queue_grid(work_grid(a.B * a.T, a.Hkv, 1), a.map.work_counters), 1, 1), dim3(kBwdThreads), lds_kv,
+        static const int resident = resident_workgroups(attn_bwd_dkv_bf16_kernel<D, HAS_DOC>, kBwdThreads, lds_kv);
+        hipLaunchKernelGGL((attn_bwd_dkv_bf16_kernel<D, HAS_DOC>), dim3(queue_grid(work_grid(a.B * a.T, a.Hkv, 1), a.map.work_counters, resident), 1, 1), dim3(kBwdThreads), lds_kv,
                            st, a);
         rc = check_launch("attn_bwd_dkv_bf16_kernel");
     }

@@ -16,6 +16,10 @@
 #include "common.h"
 #include "mfma.h"
 
+#ifndef MA_PAIR_MIN_D
+#define MA_PAIR_MIN_D 256  /* below that the one-head kernel fits two workgroups per compute unit, which beats sharing K/V fragments */
+#endif
+
 namespace ma {
 
 constexpr int kFwdThreads = 256;
@@ -315,8 +319,9 @@ static int fwd_dd(const AttnArgs& a, hipStream_t st) {
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return fail(MA_ERR_LAUNCH, "hipFuncSetAttribute(attn_fwd_bf16, %zu): %s", lds, hipGetErrorString(e));
     }
-    hipLaunchKernelGGL((attn_fwd_bf16_kernel<D, HAS_DOC>), dim3(queue_grid(work_grid(a.B * a.T, a.Hkv, a.Hq / a.Hkv), a.map.work_counters), 1, 1), dim3(kFwdThreads), lds,
-                       st, a);
+    static const int resident = resident_workgroups(attn_fwd_bf16_kernel<D, HAS_DOC>, kFwdThreads, lds);
+    hipLaunchKernelGGL((attn_fwd_bf16_kernel<D, HAS_DOC>), dim3(queue_grid(work_grid(a.B * a.T, a.Hkv, a.Hq / a.Hkv), a.map.work_counters, resident), 1, 1),
+                       dim3(kFwdThreads), lds, st, a);
     return check_launch("attn_fwd_bf16_kernel");
 }
 
@@ -327,7 +332,7 @@ static int fwd_d(const AttnArgs& a, hipStream_t st) {
 
 int launch_attn_fwd_bf16(const AttnArgs& a, hipStream_t st) {
     // query heads that share a kv head are processed in pairs when they come in pairs
-    if ((a.Hq / a.Hkv) % 2 == 0) return launch_attn_fwd_pair_bf16(a, st);
+    if ((a.Hq / a.Hkv) % 2 == 0 && a.D >= MA_PAIR_MIN_D) return launch_attn_fwd_pair_bf16(a, st);
     switch (a.D) {
         case 64: return fwd_d<64>(a, st);
         case 128: return fwd_d<128>(a, st);

@@ -345,7 +345,9 @@ static int pair_dd(const AttnArgs& a, hipStream_t st) {
         if (e != hipSuccess) return fail(MA_ERR_LAUNCH, "hipFuncSetAttribute(attn_fwd_pair_bf16, %zu): %s", lds, hipGetErrorString(e));
     }
     const int GP = a.Hq / a.Hkv / 2;
-    hipLaunchKernelGGL((attn_fwd_pair_bf16_kernel<D, HAS_DOC>), dim3(queue_grid(work_grid(a.B * a.T, a.Hkv, GP), a.map.work_counters), 1, 1), dim3(kPairThreads), lds, st, a);
+    static const int resident = resident_workgroups(attn_fwd_pair_bf16_kernel<D, HAS_DOC>, kPairThreads, lds);
+    hipLaunchKernelGGL((attn_fwd_pair_bf16_kernel<D, HAS_DOC>), dim3(queue_grid(work_grid(a.B * a.T, a.Hkv, GP), a.map.work_counters, resident), 1, 1),
+                       dim3(kPairThreads), lds, st, a);
     return check_launch("attn_fwd_pair_bf16_kernel");
 }
 

@@ -186,10 +186,17 @@ inline int compute_units() {
     }
     return c;
 }
-inline int queue_grid(int total_ids, const int32_t* counters) {
+// as many workgroups as the device holds at once (`resident` per compute unit, from the occupancy query)
+inline int queue_grid(int total_ids, const int32_t* counters, int resident = 1) {
     if (!counters) return total_ids;
-    const int cus = compute_units();
-    return total_ids < cus ? total_ids : cus;
+    const int slots = compute_units() * (resident < 1 ? 1 : resident);
+    return total_ids < slots ? total_ids : slots;
+}
+template <typename K>
+inline int resident_workgroups(K kernel, int threads, size_t lds_bytes) {
+    int n = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, (const void*)kernel, threads, lds_bytes) != hipSuccess || n < 1) n = 1;
+    return n;
 }
 
 // Walks `reps` times over the concatenation of two tile lists (partial tiles, then full tiles) of a
