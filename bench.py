@@ -73,7 +73,7 @@ def cpu_baseline(wl, seconds_hint=20.0):
     }
 
 
-def flex_gpu_baseline(wl, q, k, steps=10, warmup=3):
+def flex_gpu_baseline(wl, q, k, steps=30, warmup=10):
     """What maester runs today, on this GPU: torch's create_block_mask + torch.compile(flex_attention)
     (Inductor Triton templates; maester/models/gemma/model.py:384-396, 694-730) on the same inputs,
     driven by a restated mask mod.  Informational only: never part of the timed step, and skipped
@@ -109,8 +109,9 @@ def flex_gpu_baseline(wl, q, k, steps=10, warmup=3):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    # defaults long enough for the clocks to settle: the first ~50 steps of a cold GPU run 5-8 % slower
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--workload", default="c2")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-flex-baseline", action="store_true",
