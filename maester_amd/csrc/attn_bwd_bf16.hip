@@ -524,15 +524,22 @@ __device__ __forceinline__ void attn_bwd_dq_bf16_item(KernArgs& a, const int wg_
             const uint32_t pdst = nb ? vdst : kdst, psb = nb ? vsb : ksb;
             constexpr int kEvery = (2 * KK) / decltype(sk)::PER;
             static_assert(kEvery >= 1, "pacing");
-            auto pace_hook = [&](auto idx) {
+            // S^T = K Q^T, then dP^T = V dO^T, for 32 kv rows x the wave's 32 q rows (lane owns one q
+            // row).  The two products run one after the other so that the exponentials of S^T (a
+            // quarter-rate instruction each) are taken in the shadow of the dP^T MFMAs: one value
+            // per MFMA, from the second MFMA after S^T is complete; what does not fit follows the chain.
+            f32x16 s, dp;
+            constexpr int kFirstExp = KK + 2, kHooked = (2 * KK - kFirstExp) < 16 ? (2 * KK - kFirstExp) : 16;
+            auto chain_hook = [&](auto idx) {
                 constexpr int i = decltype(idx)::value;
                 if constexpr (i % kEvery == kEvery - 1) sk.template issue_one<i / kEvery>(psrc, pdst, w, pace, psb);
+                if constexpr (i >= kFirstExp && i - kFirstExp < 16) s[i - kFirstExp] = fast_exp2(s[i - kFirstExp] * sl2 - lse2);
             };
-
-            // S^T = K Q^T and dP^T = V dO^T for 32 kv rows x the wave's 32 q rows (lane owns one q row)
-            f32x16 s, dp;
             const uint32_t roff = (uint32_t)(32 * nb * TL::kPitch);
-            rowfrag_gemm2<D, kBPipe, false, true>(lds_addr(Ks) + rbase + roff, qf, s, lds_addr(Vs) + rbase + roff, gf, dp, pace_hook);
+            rowfrag_gemm2<D, kBPipe, false, true, decltype(chain_hook)&, true>(lds_addr(Ks) + rbase + roff, qf, s, lds_addr(Vs) + rbase + roff, gf, dp,
+                                                                                 chain_hook);
+#pragma unroll
+            for (int v = kHooked; v < 16; ++v) s[v] = fast_exp2(s[v] * sl2 - lse2);
 
             bf16x8 dsf[2];
             const int qrel = q - kb0 - 4 * hh;                     // d = q - kv = qrel - (8*(v/4) + v%4)
@@ -553,7 +560,7 @@ __device__ __forceinline__ void attn_bwd_dq_bf16_item(KernArgs& a, const int wg_
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         const int v = 4 * g4 + e;
-                        float p = fast_exp2(s[v] * sl2 - lse2);
+                        float p = s[v];  // exp2(S^T * scale - lse) by now
                         if (MASKED) {
                             bool ok = (t0 - (unsigned)(8 * g4 + e) <= span) & some;
                             if (HAS_DOC) ok = ok & (ids[e] == docq);

@@ -6,7 +6,10 @@ gfx950 assembly (``python -m maester_amd.isa_check`` or ``check_all()``):
 
 1. **MFMA results.**  No hazard padding is inserted around ``asm`` MFMAs: between an MFMA and the
    next fence (``s_nop`` of 16 wait states), branch, label or barrier, no compiler-scheduled vector
-   or memory instruction may read or write a register that an MFMA of the current chain writes.
+   or memory instruction may read or write a register that one of the last two MFMAs wrote (an
+   8-pass MFMA's result needs 11 wait states before the vector ALU may touch it; a register that
+   two later MFMAs, 16 passes, have left alone is safe -- the kernels use that to work on a finished
+   accumulator from the hooks of the chain that follows).
 2. **Scalar loads in flight.**  An ``asm`` ``s_load`` returns its data some hundred cycles later,
    into the physical registers it named.  Until the next ``s_waitcnt lgkmcnt(0)`` nothing may read
    or write those registers: a spill of the (not yet loaded) tuple, followed by a reuse of the
@@ -43,7 +46,7 @@ def check_assembly(asm: str) -> tuple[list[str], dict]:
     for m in re.finditer(r"^(_ZN2ma\w+):[^\n]*\n(.*?)s_endpgm", asm, re.S | re.M):
         name, body = m.group(1), m.group(2).split("\n")
         in_asm = False
-        chain = set()      # vector registers written by MFMAs of the current chain
+        chain = {}         # vector register written by an MFMA of the current chain -> MFMAs issued since
         pending = set()    # scalar registers of asm loads that have not been waited for
         n_mfma = n_sload = 0
         for i, ln in enumerate(body):
@@ -57,7 +60,7 @@ def check_assembly(asm: str) -> tuple[list[str], dict]:
             if not t or t.startswith(";"):
                 continue
             if t.startswith((".LBB", "s_cbranch", "s_branch", "s_barrier")):
-                chain = set()
+                chain = {}
                 if pending and t.startswith(("s_cbranch", "s_branch")):
                     # a branch between an asm load and its wait: the linear scan no longer follows the program
                     pass
@@ -65,7 +68,7 @@ def check_assembly(asm: str) -> tuple[list[str], dict]:
             mm = re.match(r"s_nop (\d+)", t)
             if mm:
                 if int(mm.group(1)) >= 15:
-                    chain = set()
+                    chain = {}
                 continue
             ops = t.split(None, 1)[1] if " " in t else ""
             if t.startswith("s_waitcnt"):
@@ -79,13 +82,14 @@ def check_assembly(asm: str) -> tuple[list[str], dict]:
             if in_asm:
                 if t.startswith("v_mfma"):
                     n_mfma += 1
-                    chain |= _regs(ops.split(",")[0], "va")
+                    chain = {r: age + 1 for r, age in chain.items() if age + 1 < 2}
+                    chain.update({r: 0 for r in _regs(ops.split(",")[0], "va")})
                 elif t.startswith("s_load"):
                     n_sload += 1
                     pending |= _regs(ops.split(",")[0], "s")
                 continue
             if chain and re.match(r"(v_|ds_|global_|buffer_|flat_|scratch_)", t):
-                hit = _regs(ops, "va") & chain
+                hit = _regs(ops, "va") & set(chain)
                 if hit:
                     bad.append(f"{name} line {i}: '{t}' touches in-flight MFMA result {sorted(hit)[:4]}")
         stats[name] = (n_mfma, n_sload)
