@@ -30,6 +30,9 @@ static int check_dims(const char* who, int B, int S, int Hq, int Hkv, int D) {
     if (B > 65535 || Hq > 65535) return fail(MA_ERR_BAD_ARG, "%s: B=%d / Hq=%d exceed the grid limit 65535", who, B, Hq);
     if ((int64_t)B * S > (int64_t)1 << 30) return fail(MA_ERR_BAD_ARG, "%s: B*S=%lld too large", who, (long long)B * S);
     if (D != 64 && D != 128 && D != 256) return fail(MA_ERR_UNSUPPORTED, "%s: head_dim %d not in {64,128,256}", who, D);
+    // the attention kernels keep a step as one word: 24 bits of row number, 5 bits of query head within its group
+    if (S >= (1 << 24)) return fail(MA_ERR_UNSUPPORTED, "%s: S=%d is 2^24 or more", who, S);
+    if (Hq / Hkv > 32) return fail(MA_ERR_UNSUPPORTED, "%s: %d query heads per kv head (at most 32)", who, Hq / Hkv);
     return MA_OK;
 }
 

@@ -87,6 +87,8 @@ def test_attention_argument_errors():
     assert fwd(mp=_map(False)) == _lib.MA_ERR_BAD_ARG and "tile map" in _err()
     assert fwd(causal=3) == _lib.MA_ERR_BAD_ARG
     assert fwd(B=0) == _lib.MA_ERR_BAD_ARG
+    assert fwd(S=1 << 24) == _lib.MA_ERR_UNSUPPORTED and "2^24" in _err()
+    assert fwd(Hq=66, Hkv=2) == _lib.MA_ERR_UNSUPPORTED and "per kv head" in _err()
     # backward: workspace too small, invalid stages
     rc = L.ma_attn_bwd(r(t), r(t), r(t), r(t), r(t), 0x1000, r(t), r(t), r(t), r(m), None, 1, -1, 0.1, 0x1000, 16, 1,
                        1, 256, 4, 2, 256, None)
