@@ -103,9 +103,25 @@ class GemmaAttention(nn.Module):
         else:
             theta = wl.get("global", 10_000)
             factor = (config.rope_scaling or {}).get("factor", 1) if config.rope_scaling else 1.0
-        cos, sin = precompute_rope_tables(self.head_dim, 2 * config.max_seq_len, theta, factor)
-        self.register_buffer("rope_cos", cos, persistent=False)
-        self.register_buffer("rope_sin", sin, persistent=False)
+        # kept out of the module's buffers on purpose: ``module.to(torch.bfloat16)`` must not round the
+        # tables (the reference's table is complex64 whatever the dtype of the weights)
+        self._rope_cpu = precompute_rope_tables(self.head_dim, 2 * config.max_seq_len, theta, factor)
+        self._rope_dev: dict = {}
+
+    def _rope(self, device) -> tuple:
+        device = torch.device(device)
+        if device not in self._rope_dev:
+            self._rope_dev[device] = tuple(t.to(device) for t in self._rope_cpu)
+        return self._rope_dev[device]
+
+    @property
+    def rope_cos(self) -> torch.Tensor:
+        """fp32 ``[2*max_seq_len, head_dim/2]`` on the device of the weights."""
+        return self._rope(self.qkv_proj.weight.device)[0]
+
+    @property
+    def rope_sin(self) -> torch.Tensor:
+        return self._rope(self.qkv_proj.weight.device)[1]
 
     def set_backend(self, backend: str) -> None:
         if backend not in {"flex", "naive", "hip"}:
