@@ -95,6 +95,17 @@ size_t ma_tile_map_workspace_bytes(int B, int S);
 int ma_tile_map_build(const int64_t* document_ids, int B, int S, int causal, int64_t window,
                       const ma_tile_map* out, void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---- ids of packed rows ----------------------------------------------------------------------------
+ * Replaces PackedSFTDataset._generate_position_ids / _generate_document_ids
+ * (maester/sft/packed_dataset.py:138-185) and their stacking in packed_collate_fn
+ * (maester/sft/dataset.py:198-220), on the device: the i-th boundary (start, length) of row b covers
+ * tokens [start, min(start + length, S)) with positions 0, 1, ... and document id i; a later
+ * boundary overwrites an earlier one; uncovered tokens (padding) get position 0 and id -1.
+ * starts, lengths: int32 [B, max_docs] (row-major, entries past counts[b] ignored); counts: int32 [B].
+ * position_ids, document_ids: int64 [B,S] outputs; either may be NULL. */
+int ma_packed_ids_build(const int32_t* starts, const int32_t* lengths, const int32_t* counts, int B, int max_docs, int S,
+                        int64_t* position_ids, int64_t* document_ids, void* stream);
+
 /* ---- fused QK-RMSNorm + RoPE prologue ------------------------------------------------------------
  * Replaces query_norm/key_norm (model.py:135-172, 366-368) followed by apply_rotary_emb
  * (model.py:97-106, 371-372) with the table gather by position_ids (model.py:744-747):

@@ -11,10 +11,12 @@ from .tile_map import TileMap, build_tile_map
 from .rope import precompute_rope_tables
 from .attention import (PackedDocAttention, packed_doc_attention, qk_norm_rope, doc_masked_attention)
 from .gemma_attention import GemmaAttention, GemmaAttentionConfig
-from .packed_ids import generate_position_ids, generate_document_ids, packed_collate_ids
+from .packed_ids import (generate_position_ids, generate_document_ids, packed_collate_ids, boundaries_to_tensors,
+                         device_packed_ids)
 
 __all__ = [
     "TileMap", "build_tile_map", "precompute_rope_tables", "PackedDocAttention", "packed_doc_attention",
     "qk_norm_rope", "doc_masked_attention", "GemmaAttention", "GemmaAttentionConfig",
-    "generate_position_ids", "generate_document_ids", "packed_collate_ids",
+    "generate_position_ids", "generate_document_ids", "packed_collate_ids", "boundaries_to_tensors",
+    "device_packed_ids",
 ]

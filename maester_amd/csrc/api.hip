@@ -113,6 +113,18 @@ int ma_tile_map_build(const int64_t* document_ids, int B, int S, int causal, int
     return launch_tile_map(document_ids, B, S, causal, window, *out, workspace, (hipStream_t)stream);
 }
 
+int ma_packed_ids_build(const int32_t* starts, const int32_t* lengths, const int32_t* counts, int B, int max_docs, int S,
+                        int64_t* position_ids, int64_t* document_ids, void* stream) {
+    const char* who = "ma_packed_ids_build";
+    if (B <= 0 || S <= 0) return fail(MA_ERR_BAD_ARG, "%s: B=%d and S=%d must be positive", who, B, S);
+    if (B > 65535) return fail(MA_ERR_BAD_ARG, "%s: B=%d exceeds the grid limit 65535", who, B);
+    if (max_docs < 0) return fail(MA_ERR_BAD_ARG, "%s: max_docs=%d is negative", who, max_docs);
+    if (!counts) return fail(MA_ERR_BAD_ARG, "%s: counts is NULL", who);
+    if (max_docs > 0 && (!starts || !lengths)) return fail(MA_ERR_BAD_ARG, "%s: starts / lengths are NULL", who);
+    if (!position_ids && !document_ids) return fail(MA_ERR_BAD_ARG, "%s: both outputs are NULL", who);
+    return launch_packed_ids(starts, lengths, counts, B, max_docs, S, position_ids, document_ids, (hipStream_t)stream);
+}
+
 int ma_prologue_fwd(const ma_tensor4* q_in, const ma_tensor4* k_in, const ma_tensor4* q_out, const ma_tensor4* k_out,
                     const float* q_weight, const float* k_weight, const float* rope_cos, const float* rope_sin,
                     int64_t n_pos, const int64_t* position_ids, float eps, int add_unit_offset, float* q_rstd,

@@ -43,6 +43,9 @@ int launch_prologue_bwd(const ma_tensor4& qi, const ma_tensor4& ki, const ma_ten
                         const float* q_rstd, const float* k_rstd, float* dqw, float* dkw, void* ws, int dtype,
                         int B, int S, int Hq, int Hkv, int D, hipStream_t st);
 
+int launch_packed_ids(const int32_t* starts, const int32_t* lengths, const int32_t* counts, int B, int max_docs, int S,
+                      int64_t* position_ids, int64_t* document_ids, hipStream_t st);
+
 struct AttnArgs {
     ma_tensor4 q, k, v, o, dout, dq, dk, dv;
     float* lse;

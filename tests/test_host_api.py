@@ -67,6 +67,16 @@ def test_tile_map_argument_errors():
     assert L.ma_tile_map_build(None, 1, 1024, 1, -1, ctypes.byref(m), None, 1 << 20, None) == _lib.MA_ERR_BAD_ARG
 
 
+def test_packed_ids_argument_errors():
+    L = _lib.lib()
+    ok = (0x1000, 0x1000, 0x1000)
+    assert L.ma_packed_ids_build(*ok, 0, 4, 128, 0x1000, 0x1000, None) == _lib.MA_ERR_BAD_ARG
+    assert L.ma_packed_ids_build(0x1000, 0x1000, None, 1, 4, 128, 0x1000, 0x1000, None) == _lib.MA_ERR_BAD_ARG and "counts" in _err()
+    assert L.ma_packed_ids_build(None, 0x1000, 0x1000, 1, 4, 128, 0x1000, 0x1000, None) == _lib.MA_ERR_BAD_ARG and "starts" in _err()
+    assert L.ma_packed_ids_build(*ok, 1, -1, 128, 0x1000, 0x1000, None) == _lib.MA_ERR_BAD_ARG
+    assert L.ma_packed_ids_build(*ok, 1, 4, 128, None, None, None) == _lib.MA_ERR_BAD_ARG and "outputs" in _err()
+
+
 def test_attention_argument_errors():
     L = _lib.lib()
     t, m = _t4(), _map()
