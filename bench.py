@@ -202,6 +202,19 @@ def main():
             torch.autograd.grad(o, xs + [w for w in ws_ if w is not None], wl.dout)
         t_full = time_region(full, max(K // 2, 2), 2)
 
+    # ---- sandwich RMSNorm + residual of the same model, on [B*S, model dim] (HBM roofline) -----------
+    from maester_amd.rmsnorm import rmsnorm_backward, rmsnorm_forward
+    model_dim = {"c1": 640, "c2": 2560, "c3": 2560, "c4": 3840, "c5": 4096}.get(args.workload, 2560)
+    nx = torch.randn(sp.B * sp.S, model_dim, device=dev).to(wl.xq.dtype)
+    nres, ndy = torch.randn_like(nx), torch.randn_like(nx)
+    nw = 0.1 * torch.randn(model_dim, device=dev)
+    _, nrstd = rmsnorm_forward(nx, nw, nres)
+    kn = max(K // 4, 2)
+    t_norm_f = time_region(lambda: rmsnorm_forward(nx, nw, nres), kn, max(W // 4, 1))
+    t_norm_b = time_region(lambda: rmsnorm_backward(nx, nw, nrstd, ndy), kn, max(W // 4, 1))
+    norm_bytes = 3 * nx.element_size() * nx.numel()        # x + residual in, sum out / x + dout in, dx out
+    del nx, nres, ndy
+
     # ---- the headline region: W untimed steps, then exactly K timed steps ----------------------------
     for _ in range(W):
         step()
@@ -267,6 +280,9 @@ def main():
                      "fwd_frac_hbm_peak": pro_bytes / (t_pro_f * 1e-3) / 1e9 / PEAK_HBM_GBPS,
                      "algorithmic_bytes": pro_bytes,
                      "bwd_ms": t_pro_b if has_bwd else None},
+        "sandwich_norm": {"rows": sp.B * sp.S, "dim": model_dim, "algorithmic_bytes": norm_bytes,
+                          "fwd_residual_ms": t_norm_f, "fwd_gbps": norm_bytes / (t_norm_f * 1e-3) / 1e9,
+                          "bwd_ms": t_norm_b, "bwd_gbps": norm_bytes / (t_norm_b * 1e-3) / 1e9},
         "tile_map": {"build_ms": t_map, "partial_tiles": n_partial, "full_tiles": n_full, "tiles": sp.B * T * T,
                      "skipped_tile_ratio": 1.0 - (n_partial + n_full) / float(sp.B * T * T),
                      "skipped_vs_causal": 1.0 - (n_partial + n_full) / float(sp.B * T * (T + 1) // 2)},

@@ -106,6 +106,22 @@ int ma_tile_map_build(const int64_t* document_ids, int B, int S, int causal, int
 int ma_packed_ids_build(const int32_t* starts, const int32_t* lengths, const int32_t* counts, int B, int max_docs, int S,
                         int64_t* position_ids, int64_t* document_ids, void* stream);
 
+/* ---- sandwich RMSNorms of the decoder layer ----------------------------------------------------------
+ * Replaces RMSNorm.forward (maester/models/gemma/model.py:135-172) as Gemma2DecoderLayer.forward uses
+ * it (model.py:488-508), and its autograd:
+ *   r = rsqrt(mean(x^2) + eps);  y = x * r * (add_unit_offset ? 1 + w : w)     (fp32 math)
+ *   out = residual ? residual + round(y) : y        (round = cast to the IO dtype, as the reference
+ *         does between the post-norm and `residual + hidden_states`).
+ * x, residual, out, dout, dx: contiguous [rows, dim] of dtype; weight, dweight: fp32 [dim];
+ * rstd: fp32 [rows] (forward output, may be NULL when no backward follows; backward input).
+ * The gradient of the residual input is dout itself (nothing to compute).  dim: a multiple of 8, at
+ * most 8192.  out may alias x or residual; dx may alias dout. */
+size_t ma_rmsnorm_bwd_workspace_bytes(int64_t rows, int dim);
+int ma_rmsnorm_fwd(const void* x, const void* residual, const float* weight, void* out, float* rstd, int64_t rows, int dim,
+                   float eps, int add_unit_offset, int dtype, void* stream);
+int ma_rmsnorm_bwd(const void* x, const float* weight, const float* rstd, const void* dout, void* dx, float* dweight,
+                   void* workspace, size_t workspace_bytes, int64_t rows, int dim, int add_unit_offset, int dtype, void* stream);
+
 /* ---- fused QK-RMSNorm + RoPE prologue ------------------------------------------------------------
  * Replaces query_norm/key_norm (model.py:135-172, 366-368) followed by apply_rotary_emb
  * (model.py:97-106, 371-372) with the table gather by position_ids (model.py:744-747):

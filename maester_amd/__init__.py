@@ -11,6 +11,7 @@ from .tile_map import TileMap, build_tile_map
 from .rope import precompute_rope_tables
 from .attention import (PackedDocAttention, packed_doc_attention, qk_norm_rope, doc_masked_attention)
 from .gemma_attention import GemmaAttention, GemmaAttentionConfig
+from .rmsnorm import RMSNorm, rms_norm
 from .packed_ids import (generate_position_ids, generate_document_ids, packed_collate_ids, boundaries_to_tensors,
                          device_packed_ids)
 
@@ -18,5 +19,5 @@ __all__ = [
     "TileMap", "build_tile_map", "precompute_rope_tables", "PackedDocAttention", "packed_doc_attention",
     "qk_norm_rope", "doc_masked_attention", "GemmaAttention", "GemmaAttentionConfig",
     "generate_position_ids", "generate_document_ids", "packed_collate_ids", "boundaries_to_tensors",
-    "device_packed_ids",
+    "device_packed_ids", "RMSNorm", "rms_norm",
 ]

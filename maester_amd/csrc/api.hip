@@ -113,6 +113,44 @@ int ma_tile_map_build(const int64_t* document_ids, int B, int S, int causal, int
     return launch_tile_map(document_ids, B, S, causal, window, *out, workspace, (hipStream_t)stream);
 }
 
+static int check_norm(const char* who, const void* x, const float* weight, int64_t rows, int dim, int dtype) {
+    MA_TRY(check_dtype(who, dtype));
+    if (rows <= 0 || rows > ((int64_t)1 << 31) - 1) return fail(MA_ERR_BAD_ARG, "%s: rows=%lld out of range", who, (long long)rows);
+    if (dim <= 0 || dim % 8 != 0 || dim > 8192)
+        return fail(MA_ERR_UNSUPPORTED, "%s: dim=%d must be a multiple of 8, at most 8192", who, dim);
+    if (!x || !weight) return fail(MA_ERR_BAD_ARG, "%s: x / weight is NULL", who);
+    if (((uintptr_t)x & 15) != 0 || ((uintptr_t)weight & 15) != 0) return fail(MA_ERR_BAD_ARG, "%s: x / weight not 16-byte aligned", who);
+    return MA_OK;
+}
+
+size_t ma_rmsnorm_bwd_workspace_bytes(int64_t rows, int dim) {
+    if (rows <= 0 || dim <= 0) return 0;
+    return (size_t)rmsnorm_bwd_blocks(rows) * dim * sizeof(float);
+}
+
+int ma_rmsnorm_fwd(const void* x, const void* residual, const float* weight, void* out, float* rstd, int64_t rows, int dim,
+                   float eps, int add_unit_offset, int dtype, void* stream) {
+    const char* who = "ma_rmsnorm_fwd";
+    MA_TRY(check_norm(who, x, weight, rows, dim, dtype));
+    if (!out || ((uintptr_t)out & 15) != 0) return fail(MA_ERR_BAD_ARG, "%s: out is NULL or not 16-byte aligned", who);
+    if (residual && ((uintptr_t)residual & 15) != 0) return fail(MA_ERR_BAD_ARG, "%s: residual not 16-byte aligned", who);
+    if (!(eps >= 0.f)) return fail(MA_ERR_BAD_ARG, "%s: eps must be >= 0", who);
+    return launch_rmsnorm_fwd(x, residual, weight, out, rstd, rows, dim, eps, add_unit_offset ? 1 : 0, dtype, (hipStream_t)stream);
+}
+
+int ma_rmsnorm_bwd(const void* x, const float* weight, const float* rstd, const void* dout, void* dx, float* dweight,
+                   void* workspace, size_t workspace_bytes, int64_t rows, int dim, int add_unit_offset, int dtype, void* stream) {
+    const char* who = "ma_rmsnorm_bwd";
+    MA_TRY(check_norm(who, x, weight, rows, dim, dtype));
+    if (!rstd || !dout || !dx || !dweight) return fail(MA_ERR_BAD_ARG, "%s: rstd / dout / dx / dweight is NULL", who);
+    if ((((uintptr_t)dout | (uintptr_t)dx) & 15) != 0) return fail(MA_ERR_BAD_ARG, "%s: dout / dx not 16-byte aligned", who);
+    if (!workspace || workspace_bytes < ma_rmsnorm_bwd_workspace_bytes(rows, dim))
+        return fail(MA_ERR_BAD_ARG, "%s: workspace of %zu bytes, need %zu", who, workspace ? workspace_bytes : (size_t)0,
+                    ma_rmsnorm_bwd_workspace_bytes(rows, dim));
+    return launch_rmsnorm_bwd(x, weight, rstd, dout, dx, dweight, workspace, rows, dim, add_unit_offset ? 1 : 0, dtype,
+                              (hipStream_t)stream);
+}
+
 int ma_packed_ids_build(const int32_t* starts, const int32_t* lengths, const int32_t* counts, int B, int max_docs, int S,
                         int64_t* position_ids, int64_t* document_ids, void* stream) {
     const char* who = "ma_packed_ids_build";

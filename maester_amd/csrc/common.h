@@ -46,6 +46,12 @@ int launch_prologue_bwd(const ma_tensor4& qi, const ma_tensor4& ki, const ma_ten
 int launch_packed_ids(const int32_t* starts, const int32_t* lengths, const int32_t* counts, int B, int max_docs, int S,
                       int64_t* position_ids, int64_t* document_ids, hipStream_t st);
 
+int rmsnorm_bwd_blocks(int64_t rows);
+int launch_rmsnorm_fwd(const void* x, const void* residual, const float* weight, void* out, float* rstd, int64_t rows, int dim,
+                       float eps, int unit, int dtype, hipStream_t st);
+int launch_rmsnorm_bwd(const void* x, const float* weight, const float* rstd, const void* dout, void* dx, float* dw, void* ws,
+                       int64_t rows, int dim, int unit, int dtype, hipStream_t st);
+
 struct AttnArgs {
     ma_tensor4 q, k, v, o, dout, dq, dk, dv;
     float* lse;

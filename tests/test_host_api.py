@@ -77,6 +77,27 @@ def test_packed_ids_argument_errors():
     assert L.ma_packed_ids_build(*ok, 1, 4, 128, None, None, None) == _lib.MA_ERR_BAD_ARG and "outputs" in _err()
 
 
+def test_rmsnorm_argument_errors():
+    L = _lib.lib()
+    P_ = 0x1000
+
+    def fwd(x=P_, res=None, w=P_, out=P_, rstd=P_, rows=8, dim=256, eps=1e-6, dtype=1):
+        return L.ma_rmsnorm_fwd(x, res, w, out, rstd, rows, dim, eps, 1, dtype, None)
+
+    assert fwd(dim=100) == _lib.MA_ERR_UNSUPPORTED and "multiple of 8" in _err()
+    assert fwd(dim=16384) == _lib.MA_ERR_UNSUPPORTED
+    assert fwd(rows=0) == _lib.MA_ERR_BAD_ARG
+    assert fwd(x=None) == _lib.MA_ERR_BAD_ARG and "NULL" in _err()
+    assert fwd(out=0x1004) == _lib.MA_ERR_BAD_ARG and "aligned" in _err()
+    assert fwd(dtype=9) == _lib.MA_ERR_BAD_ARG
+    assert fwd(eps=-1.0) == _lib.MA_ERR_BAD_ARG
+    assert L.ma_rmsnorm_bwd_workspace_bytes(0, 256) == 0
+    rc = L.ma_rmsnorm_bwd(P_, P_, P_, P_, P_, P_, P_, 8, 64, 256, 1, 1, None)
+    assert rc == _lib.MA_ERR_BAD_ARG and "workspace" in _err()
+    rc = L.ma_rmsnorm_bwd(P_, P_, None, P_, P_, P_, P_, 1 << 30, 64, 256, 1, 1, None)
+    assert rc == _lib.MA_ERR_BAD_ARG and "rstd" in _err()
+
+
 def test_attention_argument_errors():
     L = _lib.lib()
     t, m = _t4(), _map()
