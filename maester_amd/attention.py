@@ -202,6 +202,16 @@ class _DocMaskedAttention(torch.autograd.Function):
         return dq, dk, dv, None, None, None, None, None
 
 
+# What the autograd Function keeps for its backward, beyond its inputs (which autograd holds anyway):
+#   "all"        q, k after the prologue, the output, LSE, the norms' rstd -- nothing is redone
+#   "attention"  the output and LSE only; the prologue (elementwise, one pass) is redone.  This is
+#                what the reference's op-level selective checkpointing keeps: outputs of matmuls and
+#                attention, everything elementwise recomputed (maester/parallelisms/parallelize_gemma.py:181-232)
+#   "inputs"     nothing; prologue and attention forward are redone (full checkpointing of the op,
+#                parallelize_gemma.py:195-196, without re-running the surrounding module)
+SAVE_POLICIES = ("all", "attention", "inputs")
+
+
 class PackedDocAttention(torch.autograd.Function):
     """QK-RMSNorm -> RoPE -> document-masked GQA attention, forward and backward in HIP.
 
@@ -214,36 +224,48 @@ class PackedDocAttention(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, xq, xk, xv, q_norm_w, k_norm_w, rope_cos, rope_sin, position_ids, document_ids, scale,
-                causal=True, sliding_window=None, eps=1e-6, tile_map=None):
+                causal=True, sliding_window=None, eps=1e-6, tile_map=None, save="all"):
+        if save not in SAVE_POLICIES:
+            raise ValueError(f"save={save!r}: expected one of {SAVE_POLICIES}")
         B, S = xq.shape[0], xq.shape[1]
         tile_map = _resolve_map(tile_map, document_ids, B, S, causal, sliding_window, xq.device)
         q, k, q_rstd, k_rstd = prologue_forward(xq, xk, q_norm_w, k_norm_w, rope_cos, rope_sin, position_ids, eps,
                                                 True)
         out, lse = attention_forward(q, k, xv, tile_map, document_ids, scale, causal, sliding_window)
-        ctx.save_for_backward(xq, xk, xv, q_norm_w, k_norm_w, rope_cos, rope_sin, position_ids, document_ids, q, k,
-                              out, lse, q_rstd, k_rstd)
-        ctx.tile_map, ctx.scale, ctx.causal, ctx.window = tile_map, scale, causal, sliding_window
+        kept = {"all": (q, k, out, lse, q_rstd, k_rstd), "attention": (out, lse), "inputs": ()}[save]
+        ctx.save_for_backward(xq, xk, xv, q_norm_w, k_norm_w, rope_cos, rope_sin, position_ids, document_ids, *kept)
+        ctx.tile_map, ctx.scale, ctx.causal, ctx.window, ctx.eps, ctx.save = tile_map, scale, causal, sliding_window, eps, save
         return out
 
     @staticmethod
     def backward(ctx, dout):
-        (xq, xk, xv, q_w, k_w, cos, sin, position_ids, document_ids, q, k, out, lse, q_rstd,
-         k_rstd) = ctx.saved_tensors
+        xq, xk, xv, q_w, k_w, cos, sin, position_ids, document_ids = ctx.saved_tensors[:9]
+        kept = ctx.saved_tensors[9:]
+        if ctx.save == "all":
+            q, k, out, lse, q_rstd, k_rstd = kept
+        else:  # the prologue is one HBM-bound pass: cheaper to redo than to keep q and k
+            q, k, q_rstd, k_rstd = prologue_forward(xq, xk, q_w, k_w, cos, sin, position_ids, ctx.eps, True)
+            if ctx.save == "attention":
+                out, lse = kept
+            else:
+                out, lse = attention_forward(q, k, xv, ctx.tile_map, document_ids, ctx.scale, ctx.causal, ctx.window)
         dq, dk, dv = attention_backward(q, k, xv, out, dout, lse, ctx.tile_map, document_ids, ctx.scale, ctx.causal,
                                         ctx.window)
         dxq, dxk, dqw, dkw = prologue_backward(xq, xk, dq, dk, q_w, k_w, cos, sin, position_ids, q_rstd, k_rstd, True,
                                                inplace=True)
         return (dxq, dxk, dv, _wgrad(dqw, q_w), _wgrad(dkw, k_w), None, None, None, None, None, None, None, None,
-                None)
+                None, None)
 
 
 def packed_doc_attention(xq, xk, xv, q_norm_w=None, k_norm_w=None, rope_cos=None, rope_sin=None, position_ids=None,
-                         document_ids=None, scale=None, causal=True, sliding_window=None, eps=1e-6, tile_map=None):
-    """Keyword-friendly wrapper of ``PackedDocAttention.apply``; ``scale`` defaults to ``D**-0.5``."""
+                         document_ids=None, scale=None, causal=True, sliding_window=None, eps=1e-6, tile_map=None,
+                         save="all"):
+    """Keyword-friendly wrapper of ``PackedDocAttention.apply``; ``scale`` defaults to ``D**-0.5``;
+    ``save`` picks what is kept for the backward (``SAVE_POLICIES``)."""
     if scale is None:
         scale = xq.shape[-1] ** -0.5
     return PackedDocAttention.apply(xq, xk, xv, q_norm_w, k_norm_w, rope_cos, rope_sin, position_ids, document_ids,
-                                    float(scale), bool(causal), sliding_window, float(eps), tile_map)
+                                    float(scale), bool(causal), sliding_window, float(eps), tile_map, save)
 
 
 def qk_norm_rope(xq, xk, q_norm_w, k_norm_w, rope_cos, rope_sin, position_ids=None, eps=1e-6, add_unit_offset=True):

@@ -96,6 +96,7 @@ class GemmaAttention(nn.Module):
         self.attn_type = attn_type
         self.sliding_window_size = config.sliding_window_size
         self.attention_backend = "hip"
+        self.saved_for_backward = "all"   # see maester_amd.attention.SAVE_POLICIES
         # RoPE tables (model.py:588-623): 2*max_seq_len rows; scaling factor on the global table only
         wl = config.rope_wave_length or {}
         if attn_type == "local_sliding":
@@ -152,6 +153,6 @@ class GemmaAttention(nn.Module):
             self.key_norm.weight if self.key_norm is not None else None,
             self.rope_cos, self.rope_sin, step.position_ids, step.document_ids, self.scaling,
             causal=True, sliding_window=int(self.sliding_window_size) if use_local else None, eps=self.eps,
-            tile_map=tile_map)
+            tile_map=tile_map, save=self.saved_for_backward)
         out = out.view(batch_size, input_len, -1)   # already [B,S,Hq*D]: no transposed copy
         return self.o_proj(out)

@@ -221,6 +221,22 @@ def test_full_size_backward_slices(gpu, name):
         torch.cuda.empty_cache()
 
 
+def test_saved_tensor_policies_give_identical_gradients(gpu):
+    """Keeping everything, keeping only the attention output and LSE, or keeping nothing for the
+    backward changes what is recomputed, not a bit of the result (the kernels are deterministic)."""
+    from maester_amd.attention import SAVE_POLICIES
+    wl = workloads.make("c2", B=2, S=1536).to(gpu)
+    grads = {}
+    for policy in SAVE_POLICIES:
+        leaves = [t.clone().requires_grad_() for t in (wl.xq, wl.xk, wl.xv, wl.q_w, wl.k_w)]
+        out = packed_doc_attention(*leaves, wl.cos, wl.sin, wl.position_ids, wl.document_ids, wl.scale, save=policy)
+        grads[policy] = (out.detach(),) + torch.autograd.grad(out, leaves, wl.dout)
+    for policy in SAVE_POLICIES[1:]:
+        assert all(torch.equal(a, b) for a, b in zip(grads["all"], grads[policy])), policy
+    with pytest.raises(ValueError):
+        packed_doc_attention(wl.xq, wl.xk, wl.xv, wl.q_w, wl.k_w, wl.cos, wl.sin, wl.position_ids, wl.document_ids, wl.scale, save="some")
+
+
 @pytest.mark.parametrize("heads", [(4, 2), (3, 3)], ids=["pair", "single"])
 def test_work_queues_give_the_same_results_and_reset_themselves(gpu, heads):
     """With work counters in the tile map the forward and dK/dV kernels run one workgroup per compute
