@@ -121,7 +121,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is measured on ONE GPU; --gpus N with N > 1 is not run "
-              "(the path shards over batch rows / kv heads with no exchange, see DESIGN.md).", file=sys.stderr)
+              "(the path shards over batch rows / kv heads with no exchange between GPUs).", file=sys.stderr)
         sys.exit(2)
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; the HIP path has no CPU fallback.", file=sys.stderr)
