@@ -10,7 +10,13 @@ gfx950 assembly (``python -m maester_amd.isa_check`` or ``check_all()``):
    8-pass MFMA's result needs 11 wait states before the vector ALU may touch it; a register that
    two later MFMAs, 16 passes, have left alone is safe -- the kernels use that to work on a finished
    accumulator from the hooks of the chain that follows).
-2. **Scalar loads in flight.**  An ``asm`` ``s_load`` returns its data some hundred cycles later,
+2. **MFMA operands.**  A fragment that the register allocator keeps in the "wrong" register file
+   is copied into place right in front of the ``asm`` MFMA that names it (``v_accvgpr_write``,
+   ``v_mov``), and the MFMA then reads a register the vector ALU wrote less than two wait states
+   earlier.  Compiler-issued MFMAs get the padding; ``asm`` ones do not and silently compute with
+   stale operands.  No ``asm`` MFMA may read, as A or B, a register that a vector-ALU instruction
+   wrote within the two preceding wait states.
+3. **Scalar loads in flight.**  An ``asm`` ``s_load`` returns its data some hundred cycles later,
    into the physical registers it named.  Until the next ``s_waitcnt lgkmcnt(0)`` nothing may read
    or write those registers: a spill of the (not yet loaded) tuple, followed by a reuse of the
    registers for something else, ends with the load overwriting that something else.
@@ -48,6 +54,7 @@ def check_assembly(asm: str) -> tuple[list[str], dict]:
         in_asm = False
         chain = {}         # vector register written by an MFMA of the current chain -> MFMAs issued since
         pending = set()    # scalar registers of asm loads that have not been waited for
+        recent = []        # (vector registers written by a VALU instruction, wait states since)
         n_mfma = n_sload = 0
         for i, ln in enumerate(body):
             t = ln.strip()
@@ -61,6 +68,7 @@ def check_assembly(asm: str) -> tuple[list[str], dict]:
                 continue
             if t.startswith((".LBB", "s_cbranch", "s_branch", "s_barrier")):
                 chain = {}
+                recent = []
                 if pending and t.startswith(("s_cbranch", "s_branch")):
                     # a branch between an asm load and its wait: the linear scan no longer follows the program
                     pass
@@ -69,6 +77,7 @@ def check_assembly(asm: str) -> tuple[list[str], dict]:
             if mm:
                 if int(mm.group(1)) >= 15:
                     chain = {}
+                recent = [(r, d + int(mm.group(1)) + 1) for r, d in recent if d + int(mm.group(1)) + 1 < 2]
                 continue
             ops = t.split(None, 1)[1] if " " in t else ""
             if t.startswith("s_waitcnt"):
@@ -79,6 +88,15 @@ def check_assembly(asm: str) -> tuple[list[str], dict]:
                 hit = _regs(ops, "s") & pending
                 if hit and not (in_asm and t.startswith("s_load")):
                     bad.append(f"{name} line {i}: '{t}' touches scalar registers of a load in flight {sorted(hit)[:4]}")
+            if in_asm and t.startswith("v_mfma"):
+                srcs = _regs(",".join(ops.split(",")[1:3]), "va")
+                for regs_written, d in recent:
+                    hit = srcs & regs_written
+                    if hit:
+                        bad.append(f"{name} line {i}: '{t}' reads {sorted(hit)[:4]} written by the vector ALU {d} wait state(s) earlier")
+            recent = [(r, d + 1) for r, d in recent if d + 1 < 2]
+            if not in_asm and t.startswith("v_") and not t.startswith(("v_cmp", "v_readlane", "v_readfirstlane")):
+                recent.append((_regs(ops.split(",")[0], "va"), 0))
             if in_asm:
                 if t.startswith("v_mfma"):
                     n_mfma += 1

@@ -23,12 +23,18 @@ _ZN2ma4demoEv: ; @demo
 """
 
 
-def test_checker_flags_both_kinds_of_hazard():
+def test_checker_flags_every_kind_of_hazard():
     bad, stats = isa_check.check_assembly(FAULTY)
     assert stats == {"_ZN2ma4demoEv": (1, 1)}
     assert len(bad) == 2 and "load in flight" in bad[0] and "MFMA result" in bad[1]
     clean = FAULTY.replace("\tv_writelane_b32 v170, s52, 9\n", "").replace("\tv_add_f32_e32 v1, v1, v20\n", "\ts_nop 15\n\tv_add_f32_e32 v1, v1, v20\n")
     assert isa_check.check_assembly(clean)[0] == []
+    # an operand copied into place right in front of the asm MFMA that reads it
+    copied = clean.replace("\t;;#ASMSTART\n\tv_mfma", "\tv_accvgpr_write_b32 a1, v40\n\t;;#ASMSTART\n\tv_mfma")
+    bad = isa_check.check_assembly(copied)[0]
+    assert len(bad) == 1 and "written by the vector ALU" in bad[0]
+    padded = copied.replace("\tv_accvgpr_write_b32 a1, v40\n", "\tv_accvgpr_write_b32 a1, v40\n\ts_nop 1\n")
+    assert isa_check.check_assembly(padded)[0] == []
 
 
 @pytest.mark.skipif(shutil.which("hipcc") is None, reason="hipcc not installed")
