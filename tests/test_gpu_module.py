@@ -64,3 +64,56 @@ def test_global_and_local_layer_share_one_steps_inputs(gpu):
         got = (attn.qkv_proj.weight.grad, attn.o_proj.weight.grad, attn.query_norm.weight.grad, attn.key_norm.weight.grad)
         for name, g, leaf in zip(("qkv_proj", "o_proj", "query_norm", "key_norm"), got, leaves):
             assert rel_l2(g.float().cpu(), leaf.grad) <= 2e-2, (kind, name, rel_l2(g.float().cpu(), leaf.grad))
+
+
+def _reference_layer(layer, h, step, window):
+    """One decoder layer in fp32 on the CPU: the oracle's norm and attention path, torch GEMMs."""
+    from oracle import prologue as P
+
+    def w(mod):
+        return mod.weight.detach().float().cpu()
+    a = layer.self_attn
+    B, S, _ = h.shape
+    x = P.rms_norm(h, w(layer.input_layernorm))
+    qkv = x @ w(a.qkv_proj).t()
+    xq, xk, xv = qkv.split([a.q_size, a.kv_size, a.kv_size], dim=-1)
+    o = A.full_path(xq.view(B, S, a.num_heads, a.head_dim), xk.view(B, S, a.num_kv_heads, a.head_dim),
+                    xv.view(B, S, a.num_kv_heads, a.head_dim), w(a.query_norm), w(a.key_norm), a.rope_cos.float().cpu(),
+                    a.rope_sin.float().cpu(), step.position_ids.cpu(), step.document_ids.cpu(), a.scaling, True, window)
+    h = h + P.rms_norm(o.reshape(B, S, -1) @ w(a.o_proj).t(), w(layer.post_attention_layernorm))
+    x = P.rms_norm(h, w(layer.pre_feedforward_layernorm))
+    m = layer.mlp
+    x = (torch.nn.functional.gelu(x @ w(m.gate_proj).t(), approximate="tanh") * (x @ w(m.up_proj).t())) @ w(m.down_proj).t()
+    return h + P.rms_norm(x, w(layer.post_feedforward_layernorm))
+
+
+def test_layer_stack_shares_the_steps_tile_maps(gpu):
+    """A local and a global decoder layer plus the final norm (counterpart of GemmaModel.forward,
+    maester/models/gemma/model.py:524-560) against the same stack in fp32 on the CPU."""
+    from maester_amd.gemma_layers import GemmaLayerConfig, GemmaModel
+    from oracle import prologue as P
+    torch.manual_seed(1)
+    cfg = GemmaLayerConfig(dim=256, n_heads=4, num_key_value_heads=2, head_dim=128, max_seq_len=512, sliding_window_size=64,
+                           intermediate_size=512, n_layers=2, attn_types=("local_sliding", "global"))
+    B, S = 2, 290
+    rows = [[(0, 0, 90), (1, 90, 200)], [(2, 0, 150), (3, 150, 100)]]
+    pos, doc = packed_ids.packed_collate_ids(rows, S)
+    model = GemmaModel(cfg).to(gpu).to(torch.bfloat16)
+    model.init_weights(0.06)
+    with torch.no_grad():
+        for p in model.parameters():
+            if p.dim() == 1:
+                p.copy_(0.1 * torch.randn_like(p))           # non-trivial norm weights
+    assert [l.attn_type for l in model.layers] == ["local_sliding", "global"]
+    h = torch.randn(B, S, cfg.dim).to(torch.bfloat16)
+    y = model(h.to(gpu), pos.to(gpu), doc.to(gpu))
+    step = build_step_inputs(cfg, B, S, pos.to(gpu), doc.to(gpu))
+    ref = h.float()
+    for layer, window in zip(model.layers, (64, None)):
+        ref = _reference_layer(layer, ref, step, window)
+    ref = P.rms_norm(ref, model.norm.weight.detach().float().cpu())
+    assert rel_l2(y.float().cpu(), ref) <= 2e-2, rel_l2(y.float().cpu(), ref)
+    # gradients flow to every parameter, through both layers
+    y.float().pow(2).mean().backward()
+    assert all(p.grad is not None and torch.isfinite(p.grad.float()).all() and float(p.grad.float().abs().sum()) > 0
+               for p in model.parameters())
