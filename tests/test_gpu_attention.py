@@ -115,6 +115,9 @@ BF16_CASES = [
     ("no_ids_causal", 1, 640, 2, 1, 256, None, "none"),
     ("d64", 1, 512, 2, 2, 64, None, "docs"),
     ("tiny_one_tile", 1, 50, 2, 1, 128, None, "docs"),
+    ("two_pairs_per_kv_head_d256", 1, 900, 8, 2, 256, None, "docs"),     # pair kernel, two pairs per kv head
+    ("odd_group_d256", 1, 700, 3, 1, 256, 200, "docs"),                  # one-head kernel at D = 256
+    ("mha_d256_padded", 1, 450, 2, 2, 256, None, "padded"),
 ]
 
 
