@@ -29,6 +29,8 @@ def _ids(B, S, seed, kind="docs"):
             ids[b, c:] += 1
     if kind == "padded":
         ids[:, S - S // 7:] = -1
+    if kind == "recurring":          # ids that come back later in the row: the mask only asks for equality
+        ids = ids % 3
     return torch.from_numpy(ids)
 
 
@@ -118,6 +120,8 @@ BF16_CASES = [
     ("two_pairs_per_kv_head_d256", 1, 900, 8, 2, 256, None, "docs"),     # pair kernel, two pairs per kv head
     ("odd_group_d256", 1, 700, 3, 1, 256, 200, "docs"),                  # one-head kernel at D = 256
     ("mha_d256_padded", 1, 450, 2, 2, 256, None, "padded"),
+    ("recurring_ids", 2, 1100, 4, 2, 256, None, "recurring"),
+    ("recurring_ids_window_d128", 1, 1100, 4, 1, 128, 256, "recurring"),
 ]
 
 
