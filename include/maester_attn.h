@@ -122,6 +122,27 @@ int ma_rmsnorm_fwd(const void* x, const void* residual, const float* weight, voi
 int ma_rmsnorm_bwd(const void* x, const float* weight, const float* rstd, const void* dout, void* dx, float* dweight,
                    void* workspace, size_t workspace_bytes, int64_t rows, int dim, int add_unit_offset, int dtype, void* stream);
 
+/* ---- softmax cross entropy of the fused linear + cross-entropy loss ------------------------------------
+ * Replaces the elementwise half of linear_cross_entropy(hidden.flatten(0,1), embedder_weight,
+ * labels.flatten(0,1)) (maester/models/gemma/model.py:762-769; cut-cross-entropy 25.9.3, defaults:
+ * ignore_index -100, mean over the rows that count) and of F.cross_entropy(pred.float(), labels)
+ * (train.py:258-259).  The caller forms the logits a block of rows at a time (library GEMM), calls
+ * ma_ce_rows on the block and uses what it leaves there for the two gradient GEMMs.
+ *
+ * ma_ce_valid_count: stats[0] = number of targets that count (!= ignore_index, inside [0, vocab)),
+ *   stats[1] = 1 / stats[0] (the gradient scale of the mean reduction), both fp32 on the device.
+ * ma_ce_rows: logits [rows, vocab] of dtype with `pitch` elements between rows; targets int64 [rows].
+ *   Per row: lse[row] = log sum_j exp(x_j); nll[row] = lse - x_label, 0 for a row that does not count
+ *   (natural log, fp32; either output may be NULL).  softcap > 0 replaces x by softcap*tanh(x/softcap).
+ *   With write_grad the row is overwritten by (softmax(x) - onehot(label)) * grad_scale[0] (times the
+ *   soft cap's derivative), zeros for a row that does not count; grad_scale: device fp32 or NULL (= 1).
+ * ma_ce_loss_reduce: loss[0] = (sum of nll[0..n) in a fixed order) * scale[0]; scale device fp32 or
+ *   NULL (= 1).  With scale = stats + 1 and no row that counts the loss is NaN, as torch's is. */
+int ma_ce_valid_count(const int64_t* targets, int64_t n, int64_t ignore_index, int64_t vocab, float* stats, void* stream);
+int ma_ce_rows(void* logits, int64_t pitch, const int64_t* targets, int64_t rows, int64_t vocab, int64_t ignore_index,
+               float softcap, const float* grad_scale, float* lse, float* nll, int write_grad, int dtype, void* stream);
+int ma_ce_loss_reduce(const float* nll, int64_t n, const float* scale, float* loss, void* stream);
+
 /* ---- fused QK-RMSNorm + RoPE prologue ------------------------------------------------------------
  * Replaces query_norm/key_norm (model.py:135-172, 366-368) followed by apply_rotary_emb
  * (model.py:97-106, 371-372) with the table gather by position_ids (model.py:744-747):

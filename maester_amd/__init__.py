@@ -12,6 +12,7 @@ from .rope import precompute_rope_tables
 from .attention import (PackedDocAttention, packed_doc_attention, qk_norm_rope, doc_masked_attention)
 from .gemma_attention import GemmaAttention, GemmaAttentionConfig
 from .rmsnorm import RMSNorm, rms_norm
+from .linear_ce import ce_rows, linear_cross_entropy
 from .gemma_layers import GemmaLayerConfig, GemmaMLP, Gemma2DecoderLayer, GemmaModel
 from .packed_ids import (generate_position_ids, generate_document_ids, packed_collate_ids, boundaries_to_tensors,
                          device_packed_ids)
@@ -20,5 +21,5 @@ __all__ = [
     "TileMap", "build_tile_map", "precompute_rope_tables", "PackedDocAttention", "packed_doc_attention",
     "qk_norm_rope", "doc_masked_attention", "GemmaAttention", "GemmaAttentionConfig",
     "generate_position_ids", "generate_document_ids", "packed_collate_ids", "boundaries_to_tensors",
-    "device_packed_ids", "RMSNorm", "rms_norm", "GemmaLayerConfig", "GemmaMLP", "Gemma2DecoderLayer", "GemmaModel",
+    "device_packed_ids", "RMSNorm", "rms_norm", "ce_rows", "linear_cross_entropy", "GemmaLayerConfig", "GemmaMLP", "Gemma2DecoderLayer", "GemmaModel",
 ]

@@ -151,6 +151,36 @@ int ma_rmsnorm_bwd(const void* x, const float* weight, const float* rstd, const 
                               (hipStream_t)stream);
 }
 
+int ma_ce_valid_count(const int64_t* targets, int64_t n, int64_t ignore_index, int64_t vocab, float* stats, void* stream) {
+    const char* who = "ma_ce_valid_count";
+    if (!targets || !stats) return fail(MA_ERR_BAD_ARG, "%s: targets / stats is NULL", who);
+    if (n <= 0) return fail(MA_ERR_BAD_ARG, "%s: n=%lld must be positive", who, (long long)n);
+    if (vocab <= 0 || vocab > ((int64_t)1 << 31) - 1) return fail(MA_ERR_BAD_ARG, "%s: vocab=%lld out of range", who, (long long)vocab);
+    return launch_ce_valid_count(targets, n, ignore_index, (int)vocab, stats, (hipStream_t)stream);
+}
+
+int ma_ce_rows(void* logits, int64_t pitch, const int64_t* targets, int64_t rows, int64_t vocab, int64_t ignore_index,
+               float softcap, const float* grad_scale, float* lse, float* nll, int write_grad, int dtype, void* stream) {
+    const char* who = "ma_ce_rows";
+    MA_TRY(check_dtype(who, dtype));
+    if (!logits || !targets) return fail(MA_ERR_BAD_ARG, "%s: logits / targets is NULL", who);
+    if (rows <= 0 || rows > ((int64_t)1 << 31) - 1) return fail(MA_ERR_BAD_ARG, "%s: rows=%lld out of range", who, (long long)rows);
+    if (vocab <= 0 || vocab > ((int64_t)1 << 31) - 1) return fail(MA_ERR_BAD_ARG, "%s: vocab=%lld out of range", who, (long long)vocab);
+    if (pitch < vocab) return fail(MA_ERR_BAD_ARG, "%s: pitch=%lld is below vocab=%lld", who, (long long)pitch, (long long)vocab);
+    if (!(softcap >= 0.f)) return fail(MA_ERR_BAD_ARG, "%s: softcap must be >= 0 (0 = none)", who);
+    const int elt = dtype == MA_DTYPE_BF16 ? 2 : 4;
+    if (((uintptr_t)logits & (elt - 1)) != 0) return fail(MA_ERR_BAD_ARG, "%s: logits not aligned to its element size", who);
+    return launch_ce_rows(logits, pitch, targets, rows, (int)vocab, ignore_index, softcap, grad_scale, lse, nll, write_grad ? 1 : 0,
+                          dtype, (hipStream_t)stream);
+}
+
+int ma_ce_loss_reduce(const float* nll, int64_t n, const float* scale, float* loss, void* stream) {
+    const char* who = "ma_ce_loss_reduce";
+    if (!nll || !loss) return fail(MA_ERR_BAD_ARG, "%s: nll / loss is NULL", who);
+    if (n <= 0) return fail(MA_ERR_BAD_ARG, "%s: n=%lld must be positive", who, (long long)n);
+    return launch_ce_loss_reduce(nll, n, scale, loss, (hipStream_t)stream);
+}
+
 int ma_packed_ids_build(const int32_t* starts, const int32_t* lengths, const int32_t* counts, int B, int max_docs, int S,
                         int64_t* position_ids, int64_t* document_ids, void* stream) {
     const char* who = "ma_packed_ids_build";
