@@ -106,6 +106,50 @@ def flex_gpu_baseline(wl, q, k, steps=30, warmup=10):
         return {"skipped": f"{type(e).__name__}: {str(e)[:200]}"}
 
 
+def loss_block(dev, rows, dim, vocab, dtype, with_torch):
+    """The model's last step on the same token count: fused linear + cross-entropy, loss and both gradients."""
+    import math
+
+    from maester_amd.linear_ce import ce_rows, default_chunk_rows, linear_ce_forward
+    e = torch.randn(rows, dim, device=dev).to(dtype)
+    c = (torch.randn(vocab, dim, device=dev) * (3.0 / math.sqrt(dim))).to(dtype)
+    t = torch.randint(0, vocab, (rows,), device=dev)
+    t_all = time_region(lambda: linear_ce_forward(e, c, t), 5, 2)
+    step = default_chunk_rows(vocab, e.element_size(), rows)
+    blk = torch.mm(e[:step], c.t())
+    de, dc = torch.empty_like(e[:step]), torch.empty_like(c)
+
+    def gemms():
+        torch.mm(e[:step], c.t(), out=blk)
+        torch.mm(blk, c, out=de)
+        torch.mm(blk.t(), e[:step], out=dc)
+    t_gemm = time_region(gemms, 5, 2)
+    torch.mm(e[:step], c.t(), out=blk)
+    t_rows = time_region(lambda: ce_rows(blk, t[:step]), 10, 3)
+    flops = 6.0 * rows * vocab * dim
+    row_bytes = 2 * e.element_size() * step * vocab
+    out = {"rows": rows, "dim": dim, "vocab": vocab, "rows_per_block": step, "fwd_bwd_ms": t_all,
+           "useful_flops": flops, "tflops": flops / (t_all * 1e-3) / 1e12,
+           "library_gemms_ms_per_block": t_gemm, "library_gemm_tflops": 6.0 * step * vocab * dim / (t_gemm * 1e-3) / 1e12,
+           "ce_rows_kernel": {"ms_per_block": t_rows, "algorithmic_bytes": row_bytes, "gbps": row_bytes / (t_rows * 1e-3) / 1e9,
+                              "frac_hbm_peak": row_bytes / (t_rows * 1e-3) / 1e9 / PEAK_HBM_GBPS}}
+    del blk, de, dc
+    if with_torch:
+        # the reference's materialising path (train.py:258-259) with torch's own kernels on the same inputs
+        try:
+            eg, cg = e.clone().requires_grad_(), c.clone().requires_grad_()
+
+            def mat():
+                eg.grad = cg.grad = None
+                torch.nn.functional.cross_entropy((eg @ cg.t()).float(), t).backward()
+            t_mat = time_region(mat, 2, 1)
+            out["torch_materialised_fwd_bwd_ms"] = t_mat
+            out["speedup_vs_torch_materialised"] = t_mat / t_all
+        except RuntimeError as ex:       # out of memory on a smaller card
+            out["torch_materialised_error"] = str(ex)[:200]
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -116,6 +160,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-flex-baseline", action="store_true",
                     help="skip timing torch's compiled FlexAttention (the path maester runs today) on the same inputs")
+    ap.add_argument("--no-loss", action="store_true", help="skip the fused linear + cross-entropy block")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy (reference point for rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     args = ap.parse_args()
@@ -225,6 +270,9 @@ def main():
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / K
 
+    vocab = 262144 if args.workload == "c1" else 262208
+    loss = None if args.no_loss else loss_block(dev, sp.B * sp.S, model_dim, vocab, wl.xq.dtype, not args.no_flex_baseline)
+
     fl = wl.useful_flops()
     total_flops = fl["fwd_bwd"] if has_bwd else fl["fwd"]
     value = total_flops / (ms_per_step * 1e-3) / 1e12
@@ -287,6 +335,7 @@ def main():
                      "skipped_tile_ratio": 1.0 - (n_partial + n_full) / float(sp.B * T * T),
                      "skipped_vs_causal": 1.0 - (n_partial + n_full) / float(sp.B * T * (T + 1) // 2)},
         "full_autograd_function_ms": t_full,
+        "linear_cross_entropy": loss,
         "roofline": roofline,
     }
     if not args.no_flex_baseline and sp.dtype == torch.bfloat16:

@@ -25,7 +25,7 @@ MA_WORK_COUNTERS = 64
 MA_BWD_DELTA, MA_BWD_DKV, MA_BWD_DQ, MA_BWD_ALL = 1, 2, 4, 7
 
 EXPORTS = (
-    "ma_version", "ma_last_error", "ma_tile_map_workspace_bytes", "ma_tile_map_build", "ma_packed_ids_build", "ma_rmsnorm_bwd_workspace_bytes", "ma_rmsnorm_fwd", "ma_rmsnorm_bwd", "ma_ce_valid_count", "ma_ce_rows", "ma_ce_loss_reduce", "ma_prologue_fwd",
+    "ma_version", "ma_last_error", "ma_tile_map_workspace_bytes", "ma_tile_map_build", "ma_packed_ids_build", "ma_rmsnorm_bwd_workspace_bytes", "ma_rmsnorm_fwd", "ma_rmsnorm_bwd", "ma_ce_valid_count", "ma_ce_rows", "ma_ce_loss_reduce", "ma_transpose", "ma_prologue_fwd",
     "ma_prologue_bwd_workspace_bytes", "ma_prologue_bwd", "ma_attn_fwd", "ma_attn_bwd_workspace_bytes",
     "ma_attn_bwd", "ma_attn_bwd_stages",
 )
@@ -83,6 +83,8 @@ def lib() -> ctypes.CDLL:
     L.ma_ce_rows.restype = c_int
     L.ma_ce_rows.argtypes = [c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64, c_float, c_void_p, c_void_p, c_void_p, c_int,
                              c_int, c_void_p]
+    L.ma_transpose.restype = c_int
+    L.ma_transpose.argtypes = [c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p]
     L.ma_ce_loss_reduce.restype = c_int
     L.ma_ce_loss_reduce.argtypes = [c_void_p, c_int64, c_void_p, c_void_p, c_void_p]
     L.ma_rmsnorm_bwd.restype = c_int

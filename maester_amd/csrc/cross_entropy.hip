@@ -11,10 +11,10 @@
 // matrix never exists), hands the block to this kernel, which leaves the gradient in its place, and
 // feeds that to the two gradient GEMMs.
 //
-// One workgroup per row.  A Gemma row is 262 208 logits, half a megabyte, too long to keep in
-// registers: the row is read twice (running maximum and sum, then the gradient) and written once.
-// All arithmetic is fp32 in the exp2 domain; the reduction order is fixed, so results are identical
-// from run to run.
+// One workgroup per row.  A Gemma row is 262 208 logits, half a megabyte: the row is read twice
+// (running maximum and sum, then the gradient) and written once, three passes at the HBM rate.  All
+// arithmetic is fp32 in the exp2 domain; the reduction order is fixed, so results are identical from
+// run to run.
 #include <hip/hip_runtime.h>
 
 #include "common.h"
@@ -51,60 +51,67 @@ __device__ __forceinline__ void st1<uint16_t>(uint16_t* p, float v) {
     *p = *(const uint16_t*)&b;
 }
 
-// soft-capped logit in log2 units; t receives tanh(x / cap) (unused without a cap)
+// ---- arithmetic on 8 logits ------------------------------------------------------------------------
+// Everything is kept in log2 units so that an exponential is one fused multiply-add and one exp2:
+// exp(x - lse) * scale = exp2(x * log2e - (lse2 - log2 scale)).
 template <bool CAP>
-__device__ __forceinline__ float to_log2(float x, float cap, float inv_cap, float& t) {
+__device__ __forceinline__ void soft_cap8(float* v, float* dcap, float cap, float inv_cap) {
     if (CAP) {
-        t = tanhf(x * inv_cap);
-        return cap * t * kLog2e;
-    }
-    t = 0.f;
-    return x * kLog2e;
-}
-
-// VEC: the row pitch and the vocabulary allow 8-element accesses
-template <typename T, bool CAP, bool VEC>
-__global__ __launch_bounds__(kCeThreads) void ce_rows_kernel(T* __restrict__ logits, int64_t pitch,
-                                                             const int64_t* __restrict__ targets, int vocab,
-                                                             int64_t ignore_index, float cap,
-                                                             const float* __restrict__ grad_scale, float* __restrict__ lse_out,
-                                                             float* __restrict__ nll_out, int write_grad) {
-    __shared__ float s_m[kCeWaves], s_l[kCeWaves];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int64_t row = blockIdx.x;
-    T* xr = logits + row * pitch;
-    const int64_t label = targets[row];
-    const bool valid = label != ignore_index && label >= 0 && label < vocab;
-    const float inv_cap = CAP ? 1.f / cap : 0.f;
-    // read before the second pass overwrites the row
-    float x_label = 0.f;
-    if (valid && tid == 0) x_label = ld1<T>(xr + label);
-
-    const int groups = VEC ? vocab / 8 : 0;
-    float m = -INFINITY, l = 0.f;
-    for (int g = tid; g < groups; g += kCeThreads) {
-        float v[8], t;
-        ld8<T>(xr + (int64_t)g * 8, v);
-        float vm = -INFINITY;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            v[i] = to_log2<CAP>(v[i], cap, inv_cap, t);
-            vm = fmaxf(vm, v[i]);
+            const float t = tanhf(v[i] * inv_cap);
+            v[i] = cap * t;
+            dcap[i] = 1.f - t * t;
         }
-        const float mn = fmaxf(m, vm);
-        float add = 0.f;
+    }
+}
+
+// running maximum m (log2 units) and sum l of exp2(y - m)
+template <bool CAP>
+__device__ __forceinline__ void fold8(float* v, float cap, float inv_cap, float& m, float& l) {
+    float dcap[8];
+    soft_cap8<CAP>(v, dcap, cap, inv_cap);
+    float vm = fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3]));
+    vm = fmaxf(vm, fmaxf(fmaxf(v[4], v[5]), fmaxf(v[6], v[7])));
+    const float mn = fmaxf(m, vm * kLog2e);
+    float add = 0.f;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) add += exp2f(v[i] - mn);
-        l = l * exp2f(m - mn) + add;
-        m = mn;
+    for (int i = 0; i < 8; ++i) add += exp2f(fmaf(v[i], kLog2e, -mn));
+    l = l * exp2f(m - mn) + add;
+    m = mn;
+}
+__device__ __forceinline__ void fold1(float y, float& m, float& l) {
+    const float mn = fmaxf(m, y);
+    l = l * exp2f(m - mn) + exp2f(y - mn);
+    m = mn;
+}
+
+// v <- (softmax - onehot) * scale; shift = lse2 - log2(scale); label_elem < 0: the label is elsewhere
+template <bool CAP>
+__device__ __forceinline__ void grad8(float* v, float cap, float inv_cap, float shift, float scale, int label_elem) {
+    float dcap[8];
+    soft_cap8<CAP>(v, dcap, cap, inv_cap);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = exp2f(fmaf(v[i], kLog2e, -shift));
+    if (label_elem >= 0) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] -= i == label_elem ? scale : 0.f;
     }
-    for (int j = groups * 8 + tid; j < vocab; j += kCeThreads) {
-        float t;
-        const float y = to_log2<CAP>(ld1<T>(xr + j), cap, inv_cap, t);
-        const float mn = fmaxf(m, y);
-        l = l * exp2f(m - mn) + exp2f(y - mn);
-        m = mn;
+    if (CAP) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] *= dcap[i];
     }
+}
+
+template <bool CAP>
+__device__ __forceinline__ float capped(float x, float cap, float inv_cap) {
+    return CAP ? cap * tanhf(x * inv_cap) : x;
+}
+
+// combines the (m, l) of the threads of a workgroup; s_m / s_l: one slot per wave
+template <int WAVES>
+__device__ __forceinline__ float workgroup_lse2(float m, float l, float* s_m, float* s_l) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     // a thread without elements holds (-inf, 0); in a wave of such threads m - mw would be inf - inf
     const float mw = wave_max(m);
     float lw = m == -INFINITY ? 0.f : l * exp2f(m - mw);
@@ -117,33 +124,56 @@ __global__ __launch_bounds__(kCeThreads) void ce_rows_kernel(T* __restrict__ log
     __syncthreads();
     float big = s_m[0];
 #pragma unroll
-    for (int w = 1; w < kCeWaves; ++w) big = fmaxf(big, s_m[w]);
+    for (int w = 1; w < WAVES; ++w) big = fmaxf(big, s_m[w]);
     float sum = 0.f;
 #pragma unroll
-    for (int w = 0; w < kCeWaves; ++w) sum += s_l[w] * exp2f(s_m[w] - big);
-    const float lse2 = big + log2f(sum);
+    for (int w = 0; w < WAVES; ++w) sum += s_l[w] * exp2f(s_m[w] - big);
+    return big + log2f(sum);
+}
+
+// ---- rows read twice ---------------------------------------------------------------------------------
+// VEC: the row pitch and the vocabulary allow 8-element accesses
+template <typename T, bool CAP, bool VEC>
+__global__ __launch_bounds__(kCeThreads) void ce_rows_kernel(T* __restrict__ logits, int64_t pitch,
+                                                             const int64_t* __restrict__ targets, int vocab,
+                                                             int64_t ignore_index, float cap,
+                                                             const float* __restrict__ grad_scale, float* __restrict__ lse_out,
+                                                             float* __restrict__ nll_out, int write_grad) {
+    __shared__ float s_m[kCeWaves], s_l[kCeWaves];
+    const int tid = threadIdx.x;
+    const int64_t row = blockIdx.x;
+    T* xr = logits + row * pitch;
+    const int64_t label = targets[row];
+    const bool valid = label != ignore_index && label >= 0 && label < vocab;
+    const float inv_cap = CAP ? 1.f / cap : 0.f;
+    // read before the second pass overwrites the row
+    float x_label = 0.f;
+    if (valid && tid == 0) x_label = ld1<T>(xr + label);
+
+    const int groups = VEC ? vocab / 8 : 0;
+    float m = -INFINITY, l = 0.f;
+    for (int g = tid; g < groups; g += kCeThreads) {
+        float v[8];
+        ld8<T>(xr + (int64_t)g * 8, v);
+        fold8<CAP>(v, cap, inv_cap, m, l);
+    }
+    for (int j = groups * 8 + tid; j < vocab; j += kCeThreads) fold1(capped<CAP>(ld1<T>(xr + j), cap, inv_cap) * kLog2e, m, l);
+    const float lse2 = workgroup_lse2<kCeWaves>(m, l, s_m, s_l);
 
     if (tid == 0) {
-        float t;
         if (lse_out) lse_out[row] = lse2 * kLn2;
-        if (nll_out) nll_out[row] = valid ? (lse2 - to_log2<CAP>(x_label, cap, inv_cap, t)) * kLn2 : 0.f;
+        if (nll_out) nll_out[row] = valid ? (lse2 - capped<CAP>(x_label, cap, inv_cap) * kLog2e) * kLn2 : 0.f;
     }
     if (!write_grad) return;
 
     const float scale = valid ? (grad_scale ? *grad_scale : 1.f) : 0.f;
+    const float shift = lse2 - log2f(scale);
     const int label_group = valid ? (int)(label >> 3) : -1, label_elem = (int)(label & 7);
     for (int g = tid; g < groups; g += kCeThreads) {
         float v[8];
         if (valid) {
             ld8<T>(xr + (int64_t)g * 8, v);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                float t;
-                const float y = to_log2<CAP>(v[i], cap, inv_cap, t);
-                float d = exp2f(y - lse2);
-                if (g == label_group && i == label_elem) d -= 1.f;
-                v[i] = d * scale * (CAP ? 1.f - t * t : 1.f);
-            }
+            grad8<CAP>(v, cap, inv_cap, shift, scale, g == label_group ? label_elem : -1);
         } else {
 #pragma unroll
             for (int i = 0; i < 8; ++i) v[i] = 0.f;
@@ -153,11 +183,12 @@ __global__ __launch_bounds__(kCeThreads) void ce_rows_kernel(T* __restrict__ log
     for (int j = groups * 8 + tid; j < vocab; j += kCeThreads) {
         float d = 0.f;
         if (valid) {
-            float t;
-            const float y = to_log2<CAP>(ld1<T>(xr + j), cap, inv_cap, t);
-            d = exp2f(y - lse2);
-            if (j == label) d -= 1.f;
-            d *= scale * (CAP ? 1.f - t * t : 1.f);
+            const float x = ld1<T>(xr + j);
+            float t = 0.f;
+            if (CAP) t = tanhf(x * inv_cap);
+            d = exp2f(fmaf(CAP ? cap * t : x, kLog2e, -shift));
+            if (j == label) d -= scale;
+            if (CAP) d *= 1.f - t * t;
         }
         st1<T>(xr + j, d);
     }
@@ -203,6 +234,49 @@ __global__ __launch_bounds__(kCeReduceThreads) void ce_loss_reduce_kernel(const 
     if (threadIdx.x == 0) loss[0] = (float)(s_sum[0] * (scale ? (double)*scale : 1.0));
 }
 
+// ---- [rows, cols] -> [cols, rows] -----------------------------------------------------------------
+// The gradient GEMM d hidden = d logits . C runs more than twice as fast in the library when both
+// operands are contiguous along the vocabulary, so the host keeps a transposed copy of C for one call.
+// 64 x 64 tiles through LDS, 16-byte accesses on both sides where the shape allows.
+constexpr int kTrTile = 64;
+
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_kernel(const T* __restrict__ src, T* __restrict__ dst, int64_t rows, int64_t cols) {
+    constexpr int V = 16 / sizeof(T);                              // elements per 16-byte access
+    constexpr int kPerRow = kTrTile / V;                           // accesses per tile row
+    __shared__ T tile[kTrTile][kTrTile + 2];
+    const int64_t r0 = (int64_t)blockIdx.y * kTrTile, c0 = (int64_t)blockIdx.x * kTrTile;
+    const bool vec_in = cols % V == 0 && ((uintptr_t)src & 15) == 0, vec_out = rows % V == 0 && ((uintptr_t)dst & 15) == 0;
+    for (int a = threadIdx.x; a < kTrTile * kPerRow; a += 256) {
+        const int r = a / kPerRow, c = (a % kPerRow) * V;
+        if (r0 + r >= rows) continue;
+        const T* p = src + (r0 + r) * cols + c0 + c;
+        if (vec_in && c0 + c + V <= cols) {
+            const uint4 q = *(const uint4*)p;
+            const T* e = (const T*)&q;
+#pragma unroll
+            for (int i = 0; i < V; ++i) tile[r][c + i] = e[i];
+        } else {
+            for (int i = 0; i < V && c0 + c + i < cols; ++i) tile[r][c + i] = p[i];
+        }
+    }
+    __syncthreads();
+    for (int a = threadIdx.x; a < kTrTile * kPerRow; a += 256) {
+        const int c = a / kPerRow, r = (a % kPerRow) * V;           // dst row c0 + c, dst columns r0 + r ..
+        if (c0 + c >= cols) continue;
+        T* p = dst + (c0 + c) * rows + r0 + r;
+        if (vec_out && r0 + r + V <= rows) {
+            uint4 q;
+            T* e = (T*)&q;
+#pragma unroll
+            for (int i = 0; i < V; ++i) e[i] = tile[r + i][c];
+            *(uint4*)p = q;
+        } else {
+            for (int i = 0; i < V && r0 + r + i < rows; ++i) p[i] = tile[r + i][c];
+        }
+    }
+}
+
 template <typename T>
 int launch_rows(void* logits, int64_t pitch, const int64_t* targets, int64_t rows, int vocab, int64_t ignore_index, float cap,
                 const float* grad_scale, float* lse, float* nll, int write_grad, hipStream_t stream) {
@@ -230,6 +304,15 @@ int launch_ce_rows(void* logits, int64_t pitch, const int64_t* targets, int64_t 
     if (dtype == MA_DTYPE_BF16)
         return launch_rows<uint16_t>(logits, pitch, targets, rows, vocab, ignore_index, softcap, grad_scale, lse, nll, write_grad, stream);
     return launch_rows<float>(logits, pitch, targets, rows, vocab, ignore_index, softcap, grad_scale, lse, nll, write_grad, stream);
+}
+
+int launch_transpose(const void* src, void* dst, int64_t rows, int64_t cols, int dtype, hipStream_t stream) {
+    const dim3 grid((unsigned)((cols + kTrTile - 1) / kTrTile), (unsigned)((rows + kTrTile - 1) / kTrTile));
+    if (dtype == MA_DTYPE_BF16)
+        transpose_kernel<uint16_t><<<grid, 256, 0, stream>>>((const uint16_t*)src, (uint16_t*)dst, rows, cols);
+    else
+        transpose_kernel<float><<<grid, 256, 0, stream>>>((const float*)src, (float*)dst, rows, cols);
+    return check_launch("transpose_kernel");
 }
 
 int launch_ce_valid_count(const int64_t* targets, int64_t n, int64_t ignore_index, int vocab, float* stats, hipStream_t stream) {

@@ -29,8 +29,8 @@ REDUCTIONS = ("mean", "sum")
 
 
 def default_chunk_rows(vocab: int, elt: int, rows: int) -> int:
-    """Rows per block: about 2 GiB of logits, a multiple of 256."""
-    n = -(-(1 << 31) // (vocab * elt * 256)) * 256
+    """Rows per block: about 4 GiB of logits, a multiple of 256."""
+    n = -(-(1 << 32) // (vocab * elt * 256)) * 256
     return max(1, min(n, rows))
 
 
@@ -59,6 +59,19 @@ def ce_rows(logits: torch.Tensor, targets: torch.Tensor, ignore_index: int = -10
                                   1 if write_grad else 0, _lib.dtype_code(logits.dtype), _lib.current_stream(logits.device))
     _lib.check(rc)
     return lse, nll
+
+
+def transpose(x: torch.Tensor) -> torch.Tensor:
+    """``x.t().contiguous()`` of a contiguous 2-d tensor (bf16 or fp32) with the library's tile kernel."""
+    _lib.require_gpu(x, "transpose")
+    if x.dim() != 2 or not x.is_contiguous():
+        raise ValueError("transpose needs a contiguous 2-d tensor")
+    out = torch.empty(x.shape[1], x.shape[0], dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().ma_transpose(_lib.ptr(x), _lib.ptr(out), x.shape[0], x.shape[1], _lib.dtype_code(x.dtype),
+                                    _lib.current_stream(x.device))
+    _lib.check(rc)
+    return out
 
 
 def _valid_count(targets, ignore_index, vocab):
@@ -121,6 +134,9 @@ def linear_ce_forward(e, c, targets, ignore_index=-100, softcap=None, reduction=
     step = int(chunk_rows) if chunk_rows else default_chunk_rows(vocab, e.element_size(), n)
     step = max(1, min(step, n))
     block = torch.empty(step, vocab, dtype=e.dtype, device=dev)
+    # both operands of the d hidden GEMM contiguous along the vocabulary: more than twice the library's rate
+    c_t = transpose(c) if need_de else None
+    mixed = {"out_dtype": torch.float32} if e.dtype != torch.float32 else {}
     nll = torch.empty(n, dtype=torch.float32, device=dev)
     lse = torch.empty(n, dtype=torch.float32, device=dev)
     for r0 in range(0, n, step):
@@ -129,15 +145,14 @@ def linear_ce_forward(e, c, targets, ignore_index=-100, softcap=None, reduction=
         torch.mm(e_kept[r0:r1], c.t(), out=x)
         ce_rows(x, t_kept[r0:r1], ignore_index, softcap, scale, want_grad, lse=lse[r0:r1], nll=nll[r0:r1])
         if need_de:
-            torch.mm(x, c, out=de_kept[r0:r1])
+            torch.mm(x, c_t.t(), out=de_kept[r0:r1])
         if need_dc:
-            part = torch.mm(x.t(), e_kept[r0:r1])
             if n <= step:
-                dc = part
-            elif dc_acc is None:
-                dc_acc = part.float()        # several blocks: summed in fp32, rounded once at the end
+                dc = torch.mm(x.t(), e_kept[r0:r1])
+            elif dc_acc is None:             # several blocks: summed in fp32 by the GEMMs, rounded once at the end
+                dc_acc = torch.mm(x.t(), e_kept[r0:r1], **mixed)
             else:
-                dc_acc += part
+                torch.addmm(dc_acc, x.t(), e_kept[r0:r1], out=dc_acc, **mixed)
     if need_dc and dc is None:
         dc = dc_acc.to(c.dtype)
     loss = _loss_reduce(nll, scale)

@@ -12,6 +12,7 @@ import torch.nn.functional as F
 
 from conftest import max_abs, rel_l2
 from maester_amd import ce_rows, linear_cross_entropy
+from maester_amd.linear_ce import transpose
 from oracle import linear_ce as O
 
 pytestmark = pytest.mark.gpu
@@ -81,9 +82,11 @@ def test_rows_kernel_labels_out_of_range_do_not_count(gpu):
     assert float(nll[0]) > 0 and torch.all(nll[1:] == 0) and torch.all(xg[1:] == 0)
 
 
-def test_rows_kernel_bf16(gpu):
+@pytest.mark.parametrize("vocab", [512, 262208, 300000, 1003])
+def test_rows_kernel_bf16(gpu, vocab):
+    # short rows, Gemma, longer than Gemma, a ragged width (element-wise path)
     g = torch.Generator().manual_seed(2)
-    rows, vocab = 33, 262208
+    rows = 33
     x = (3 * torch.randn(rows, vocab, generator=g)).bfloat16()
     x[:, 100] += 9
     t = _targets(g, rows, vocab, 0.2)
@@ -216,3 +219,28 @@ def test_gemma_width_against_the_materialising_path_on_the_gpu(gpu):
     assert abs(float(loss) - float(ref)) <= 1e-3
     assert rel_l2(de.float(), eg.grad.cpu().float()) <= 1e-2
     assert rel_l2(dc.float(), cg.grad.cpu().float()) <= 1e-2
+
+
+@pytest.mark.parametrize("shape", [(64, 64), (262208, 96), (130, 72), (77, 13), (1, 5)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_transpose(gpu, shape, dtype):
+    x = torch.randn(*shape).to(dtype)
+    assert torch.equal(transpose(x.to(gpu)).cpu(), x.t().contiguous())
+
+
+def test_rows_kernel_bf16_softcap(gpu):
+    g = torch.Generator().manual_seed(11)
+    rows, vocab, cap = 9, 256000, 30.0
+    x = (12 * torch.randn(rows, vocab, generator=g)).bfloat16()
+    t = _targets(g, rows, vocab, 0.2)
+    xg = x.to(gpu)
+    lse, nll = ce_rows(xg, t.to(gpu), softcap=cap)
+    xd = cap * torch.tanh(x.double() / cap)
+    p = torch.softmax(xd, 1)
+    valid = t != -100
+    p[torch.arange(rows), t.clamp_min(0)] -= 1
+    p = p * valid[:, None] * (1 - torch.tanh(x.double() / cap) ** 2)
+    assert max_abs(lse.cpu(), torch.logsumexp(xd, 1)) <= 1e-4
+    want_nll = torch.where(valid, torch.logsumexp(xd, 1) - xd[torch.arange(rows), t.clamp_min(0)], torch.zeros(rows, dtype=torch.float64))
+    assert max_abs(nll.cpu(), want_nll) <= 1e-4
+    assert rel_l2(xg.cpu().float(), p) <= 4e-3
