@@ -30,7 +30,10 @@ attention.dense_attention    torch eager ``flex_attention`` on CPU, the v=-1/+1 
                              tests/test_packed_sft.py:164-212, fp64 brute-force loops on tiny
                              inputs, ``torch.autograd.gradcheck`` (backward)
 packed_ids.*                 exact expectations of tests/test_packed_sft.py:22-66
+linear_ce.linear_cross_...   ``torch.nn.functional.cross_entropy`` + autograd in fp64 (train.py:258-259),
+                             scipy ``logsumexp``, closed forms, zero row sums, central differences
 ===========================  ====================================================================
 
-No function is "parity unpinned".
+No function of the attention path is "parity unpinned".  The gradient filter of cut-cross-entropy
+(the dependency behind model.py:762-769, absent here) is not restated: "parity unpinned".
 """
