@@ -160,6 +160,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-flex-baseline", action="store_true",
                     help="skip timing torch's compiled FlexAttention (the path maester runs today) on the same inputs")
+    ap.add_argument("--no-hand-over", action="store_true",
+                    help="backward without the dS workspace: the dQ kernel recomputes S and dP")
     ap.add_argument("--no-loss", action="store_true", help="skip the fused linear + cross-entropy block")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy (reference point for rocprofv3 FETCH_SIZE/WRITE_SIZE)")
@@ -173,7 +175,8 @@ def main():
         sys.exit(3)
 
     from maester_amd import _lib, build_tile_map, packed_doc_attention, workloads
-    from maester_amd.attention import (attention_backward, attention_forward, prologue_backward, prologue_forward)
+    from maester_amd.attention import (attention_backward, attention_forward, backward_workspace_bytes, prologue_backward,
+                                       prologue_forward)
 
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
@@ -207,8 +210,9 @@ def main():
     bufs = None
     if has_bwd:
         dq, dk, dv = attention_backward(q, k, wl.xv, out, wl.dout, lse, tmap, wl.document_ids, wl.scale, True, sp.window)
-        ws = torch.empty(max(_lib.lib().ma_attn_bwd_workspace_bytes(sp.B, sp.S, sp.Hq, sp.Hkv, sp.D), 16),
-                         dtype=torch.uint8, device=dev)
+        ws_bytes = backward_workspace_bytes(sp.B, sp.S, sp.Hq, sp.Hkv, sp.D, q.dtype, False if args.no_hand_over else None)
+        hand_over = ws_bytes >= _lib.lib().ma_attn_bwd_ds_workspace_bytes(sp.B, sp.S, sp.Hq, sp.Hkv, sp.D) and q.dtype == torch.bfloat16
+        ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
         bufs = (dq, dk, dv, ws)
 
     def fwd():
@@ -231,7 +235,8 @@ def main():
         t_bwd = time_region(bwd, K, W)
         t_delta = time_region(lambda: bwd(_lib.MA_BWD_DELTA), K, W)
         t_dkv = time_region(lambda: bwd(_lib.MA_BWD_DKV), K, W)
-        t_dq = time_region(lambda: bwd(_lib.MA_BWD_DQ | _lib.MA_BWD_DELTA), K, W)   # as in the step: delta fused in
+        # as in the step: with the dS hand-over delta is a kernel of its own, otherwise it is fused into dQ
+        t_dq = time_region(lambda: bwd(_lib.MA_BWD_DQ if hand_over else _lib.MA_BWD_DQ | _lib.MA_BWD_DELTA), K, W)
         t_pro_b = time_region(
             lambda: prologue_backward(wl.xq, wl.xk, dq, dk, wl.q_w, wl.k_w, wl.cos, wl.sin, wl.position_ids, q_rstd,
                                       k_rstd), K, W)
@@ -286,7 +291,8 @@ def main():
         ("attn_fwd_pair_bf16_kernel" if (sp.Hq // sp.Hkv) % 2 == 0 and sp.D >= 256 and sp.dtype == torch.bfloat16 else "attn_fwd_bf16_kernel"):
             {"ms": t_fwd, "algorithmic_flops": 4 * base},
         "attn_bwd_dkv_bf16_kernel": {"ms": t_dkv, "algorithmic_flops": 6 * base},   # dP, dV, dK
-        "attn_bwd_dq_bf16_kernel": {"ms": t_dq, "algorithmic_flops": 2 * base},     # dQ
+        ("attn_bwd_dq_ds_bf16_kernel" if has_bwd and hand_over else "attn_bwd_dq_bf16_kernel"):
+            {"ms": t_dq, "algorithmic_flops": 2 * base},                            # dQ
     }
     for v in kern.values():
         v["tflops"] = tf(v["algorithmic_flops"], v["ms"])
@@ -321,7 +327,8 @@ def main():
         "fwd": {"ms": t_fwd, "tflops": tf(fl["fwd"], t_fwd), "pct_peak": 100 * tf(fl["fwd"], t_fwd) / PEAK_BF16_DENSE_TFLOPS},
         "bwd": None if not has_bwd else {"ms": t_bwd, "tflops": tf(fl["bwd"], t_bwd),
                                          "pct_peak": 100 * tf(fl["bwd"], t_bwd) / PEAK_BF16_DENSE_TFLOPS,
-                                         "delta_ms": t_delta, "dkv_ms": t_dkv, "dq_ms": t_dq},
+                                         "delta_ms": t_delta, "dkv_ms": t_dkv, "dq_ms": t_dq,
+                                         "ds_hand_over": bool(hand_over), "workspace_bytes": int(ws_bytes)},
         "fwd_bwd_flashattn_convention_tflops": tf(fl["fwd_bwd_flashattn_convention"], ms_per_step) if has_bwd else None,
         "kernels": kern,
         "prologue": {"fwd_ms": t_pro_f, "fwd_gbps": pro_bytes / (t_pro_f * 1e-3) / 1e9,

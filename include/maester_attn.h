@@ -194,8 +194,14 @@ int ma_attn_fwd(const ma_tensor4* q, const ma_tensor4* k, const ma_tensor4* v, c
  *   dQ = scale * dS K; dK = scale * dS^T Q; dK/dV summed over the Hq/Hkv query heads of a kv head.
  * dK and dV are produced without global atomics (one workgroup owns a kv tile and walks the q-side
  * lists), so results are run-to-run deterministic.
- * workspace: ma_attn_bwd_workspace_bytes(...) bytes (holds delta, fp32 [B,Hq,S]). */
+ * workspace: at least ma_attn_bwd_workspace_bytes(...) bytes (holds delta, fp32 [B,Hq,S]).
+ * With ma_attn_bwd_ds_workspace_bytes(...) bytes or more (bf16 only) the dK/dV kernel, which forms
+ * dS anyway, also leaves it in the workspace (bf16, one 32 KB slot per pair of tiles and query
+ * head, B*Hq*T*T slots of which only the visited ones are touched) and the dQ kernel reduces to
+ * dQ = scale * dS K instead of recomputing S and dO V^T: same results to the last bit of the
+ * bf16 dS, fewer MFMAs, for workspace that grows with T^2 (4.3 GB at B=4, S=8192, Hq=8). */
 size_t ma_attn_bwd_workspace_bytes(int B, int S, int Hq, int Hkv, int D);
+size_t ma_attn_bwd_ds_workspace_bytes(int B, int S, int Hq, int Hkv, int D);
 int ma_attn_bwd(const ma_tensor4* q, const ma_tensor4* k, const ma_tensor4* v, const ma_tensor4* out,
                 const ma_tensor4* dout, const float* lse, const ma_tensor4* dq, const ma_tensor4* dk,
                 const ma_tensor4* dv, const ma_tile_map* map, const int64_t* document_ids, int causal,
@@ -204,7 +210,9 @@ int ma_attn_bwd(const ma_tensor4* q, const ma_tensor4* k, const ma_tensor4* v, c
 
 /* ma_attn_bwd restricted to a subset of its three kernels, for callers that time or overlap them:
  * stages is a bit mask of MA_BWD_DELTA (writes delta into the workspace), MA_BWD_DKV (reads delta,
- * writes dk and dv) and MA_BWD_DQ (reads delta, writes dq).  ma_attn_bwd == all three.  No
+ * writes dk and dv) and MA_BWD_DQ (reads delta, writes dq).  ma_attn_bwd == all three.  With the
+ * larger workspace MA_BWD_DKV also writes dS and MA_BWD_DQ reads it (and no delta): a call with
+ * MA_BWD_DQ alone then needs the dS of an earlier MA_BWD_DKV call in the same workspace.  No
  * counterpart in the reference (its backward is one fused Inductor launch,
  * torch/_inductor/kernel/flex/templates/flex_backwards.py.jinja). */
 #define MA_BWD_DELTA 1

@@ -26,7 +26,7 @@ MA_BWD_DELTA, MA_BWD_DKV, MA_BWD_DQ, MA_BWD_ALL = 1, 2, 4, 7
 
 EXPORTS = (
     "ma_version", "ma_last_error", "ma_tile_map_workspace_bytes", "ma_tile_map_build", "ma_packed_ids_build", "ma_rmsnorm_bwd_workspace_bytes", "ma_rmsnorm_fwd", "ma_rmsnorm_bwd", "ma_ce_valid_count", "ma_ce_rows", "ma_ce_loss_reduce", "ma_transpose", "ma_prologue_fwd",
-    "ma_prologue_bwd_workspace_bytes", "ma_prologue_bwd", "ma_attn_fwd", "ma_attn_bwd_workspace_bytes",
+    "ma_prologue_bwd_workspace_bytes", "ma_prologue_bwd", "ma_attn_fwd", "ma_attn_bwd_workspace_bytes", "ma_attn_bwd_ds_workspace_bytes",
     "ma_attn_bwd", "ma_attn_bwd_stages",
 )
 
@@ -104,6 +104,8 @@ def lib() -> ctypes.CDLL:
                               c_int, c_int, c_int, c_void_p]
     L.ma_attn_bwd_workspace_bytes.restype = c_size_t
     L.ma_attn_bwd_workspace_bytes.argtypes = [c_int] * 5
+    L.ma_attn_bwd_ds_workspace_bytes.restype = c_size_t
+    L.ma_attn_bwd_ds_workspace_bytes.argtypes = [c_int] * 5
     L.ma_attn_bwd.restype = c_int
     L.ma_attn_bwd.argtypes = [T4, T4, T4, T4, T4, c_void_p, T4, T4, T4, TM, c_void_p, c_int, c_int64, c_float,
                               c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]

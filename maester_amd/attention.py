@@ -131,16 +131,31 @@ def attention_forward(q, k, v, tile_map: TileMap, document_ids, scale, causal=Tr
     return out, lse
 
 
+# Largest workspace the backward takes for handing dS from the dK/dV kernel to the dQ kernel (bytes);
+# above it (long sequences: the slots grow with (S/128)^2) the dQ kernel recomputes S and dP instead.
+DS_WORKSPACE_LIMIT = 24 << 30
+
+
+def backward_workspace_bytes(B, S, Hq, Hkv, D, dtype, hand_over=None) -> int:
+    """Workspace of ``attention_backward``: with room for dS when that fits ``DS_WORKSPACE_LIMIT`` (bf16 only);
+    ``hand_over`` True / False forces the choice."""
+    L = _lib.lib()
+    small, large = L.ma_attn_bwd_workspace_bytes(B, S, Hq, Hkv, D), L.ma_attn_bwd_ds_workspace_bytes(B, S, Hq, Hkv, D)
+    if hand_over is None:
+        hand_over = dtype == torch.bfloat16 and large <= DS_WORKSPACE_LIMIT
+    return large if (hand_over and dtype == torch.bfloat16) else small
+
+
 def attention_backward(q, k, v, out, dout, lse, tile_map: TileMap, document_ids, scale, causal=True, window=None,
-                       stages=_lib.MA_BWD_ALL, buffers=None):
+                       stages=_lib.MA_BWD_ALL, buffers=None, hand_over=None):
     """Returns (dq, dk, dv) as new contiguous [B,S,H,D] tensors.  ``stages`` restricts the call to
     some of its kernels (see ``ma_attn_bwd_stages``); ``buffers`` = (dq, dk, dv, workspace) reuses
-    tensors from an earlier call, which staged calls need."""
+    tensors from an earlier call, which staged calls need.  ``hand_over``: see ``backward_workspace_bytes``."""
     B, S, Hq, Hkv, D = _check_qkv(q, k, v)
     q, k, v, out, dout = (_rowmajor(t) for t in (q, k, v, out, dout))
     dev = q.device
     L = _lib.lib()
-    ws_bytes = L.ma_attn_bwd_workspace_bytes(B, S, Hq, Hkv, D)
+    ws_bytes = backward_workspace_bytes(B, S, Hq, Hkv, D, q.dtype, hand_over)
     if buffers is None:
         dq = torch.empty((B, S, Hq, D), dtype=q.dtype, device=dev)
         dk = torch.empty((B, S, Hkv, D), dtype=q.dtype, device=dev)
@@ -148,6 +163,7 @@ def attention_backward(q, k, v, out, dout, lse, tile_map: TileMap, document_ids,
         ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
     else:
         dq, dk, dv, ws = buffers
+        ws_bytes = ws.numel() * ws.element_size()
     doc = _ids(document_ids, B, S, "document_ids")
     cs = tile_map.c_struct()
     with torch.cuda.device(dev):

@@ -265,6 +265,7 @@ int ma_prologue_bwd(const ma_tensor4* q_in, const ma_tensor4* k_in, const ma_ten
 static int fill_attn(const char* who, AttnArgs& a, const ma_tensor4* q, const ma_tensor4* k, const ma_tensor4* v,
                      const ma_tensor4* out, const ma_tile_map* map, const int64_t* document_ids, int causal,
                      int64_t window, float scale, int dtype, int B, int S, int Hq, int Hkv, int D, bool bwd) {
+    a.ds = nullptr;
     MA_TRY(check_dims(who, B, S, Hq, Hkv, D));
     MA_TRY(check_dtype(who, dtype));
     MA_TRY(check_tensor(who, "q", q, dtype));
@@ -304,6 +305,15 @@ size_t ma_attn_bwd_workspace_bytes(int B, int S, int Hq, int Hkv, int D) {
     return (size_t)B * Hq * S * sizeof(float);  // delta
 }
 
+static size_t delta_bytes_aligned(int B, int S, int Hq) { return (((size_t)B * Hq * S * sizeof(float)) + 255) & ~(size_t)255; }
+
+size_t ma_attn_bwd_ds_workspace_bytes(int B, int S, int Hq, int Hkv, int D) {
+    (void)Hkv; (void)D;
+    if (B <= 0 || S <= 0 || Hq <= 0) return 0;
+    const size_t T = ((size_t)S + MA_TILE - 1) / MA_TILE;
+    return delta_bytes_aligned(B, S, Hq) + (size_t)B * Hq * T * T * MA_TILE * MA_TILE * 2;  // delta, then dS^T in bf16
+}
+
 int ma_attn_bwd(const ma_tensor4* q, const ma_tensor4* k, const ma_tensor4* v, const ma_tensor4* out,
                 const ma_tensor4* dout, const float* lse, const ma_tensor4* dq, const ma_tensor4* dk,
                 const ma_tensor4* dv, const ma_tile_map* map, const int64_t* document_ids, int causal, int64_t window,
@@ -335,6 +345,9 @@ int ma_attn_bwd_stages(const ma_tensor4* q, const ma_tensor4* k, const ma_tensor
     a.lse = (float*)lse;
     a.delta = (float*)workspace;
     a.stages = stages;
+    // a workspace large enough for dS^T selects the hand-over between the two bf16 kernels
+    if (dtype == MA_DTYPE_BF16 && workspace_bytes >= ma_attn_bwd_ds_workspace_bytes(B, S, Hq, Hkv, D))
+        a.ds = (char*)workspace + delta_bytes_aligned(B, S, Hq);
     return dtype == MA_DTYPE_BF16 ? launch_attn_bwd_bf16(a, (hipStream_t)stream)
                                   : launch_attn_bwd_f32(a, (hipStream_t)stream);
 }

@@ -87,7 +87,9 @@ __global__ __launch_bounds__(256) void attn_delta_bf16_kernel(AttnArgs a) {
 // ------------------------------------------------------------------------------------------------
 // dK / dV
 // ------------------------------------------------------------------------------------------------
-template <int D, bool HAS_DOC>
+// WRITE_DS: every 32 x 32 block of every step the workgroup walks also leaves its dS^T in a.ds (zeros
+// for a block the wave skips), for the dQ kernel that only multiplies it with K.
+template <int D, bool HAS_DOC, bool WRITE_DS>
 __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg_id) {
     using TL = Tile<D>;
     constexpr int KK = D / 16;
@@ -203,7 +205,7 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
     auto issue_g = [&](int buf) { sq.issue((const __bf16*)gsrc, Gbuf(buf), w, lane, min(BM, a.S - st.r0), a.dout.stride_s); };
     const int my_runs = decltype(sq)::runs_of(w);
     bool have = st.next();
-    int q0 = st.r0;
+    int q0 = st.r0, rep = st.rep;
     bool partial = st.partial, act0 = st.act0, act1 = st.act1;
     if (have) {
         locate();
@@ -211,6 +213,12 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
         issue_g(0);
         issue_rows();
     }
+    // where this lane's 4 x 4 values of a 32 x 32 block go: slot (b, head, q tile, kv tile j) of a.ds,
+    // row = the lane's kv row, columns q0 % 128 + 32*mb + 8*g4 + 4*hh .. +3
+    auto ds_row = [&](int head, int q_first) {
+        const size_t slot = (((size_t)b * a.Hq + head) * a.T + (q_first >> 7)) * a.T + j;
+        return (__bf16*)a.ds + slot * (kTile * kTile) + (size_t)(32 * w + r) * kTile + (q_first & (kTile - 1)) + 4 * hh;
+    };
 
     for (int n = 0; have; ++n) {
         const int cur = n & 1;
@@ -229,6 +237,7 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
         const int cq0 = q0;
         const bool cpartial = partial;
         const bool skip[BM / 32] = {!act0, !act1};  // blocks in which this wave has nothing to do
+        __bf16* ds_out = WRITE_DS ? ds_row(hk * G + rep, cq0) : nullptr;
         have = st.next();
         // The tile loads of the next step are spread over this step's first MFMA chains, one run
         // every few MFMAs (Q tile in the first 32-row block, dO tile in the second): issued in one
@@ -237,6 +246,7 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
         int pace = 0;
         if (have) {
             q0 = st.r0;
+            rep = st.rep;
             partial = st.partial;
             act0 = st.act0;
             act1 = st.act1;
@@ -254,7 +264,13 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
 #pragma unroll 1
         for (int mb = 0; mb < BM / 32; ++mb) {
             const int qb0 = cq0 + 32 * mb;
-            if (mb ? skip[1] : skip[0]) continue;
+            if (mb ? skip[1] : skip[0]) {
+                if (WRITE_DS) {
+#pragma unroll
+                    for (int g4 = 0; g4 < 4; ++g4) *(uint2*)(ds_out + 32 * mb + 8 * g4) = make_uint2(0, 0);
+                }
+                continue;
+            }
             const __bf16* psrc = (const __bf16*)(mb ? gsrc : qsrc);
             const uint32_t pdst = mb ? gdst : qdst, psb = mb ? gsb : qsb;
             constexpr int kEvery = (2 * KK) / decltype(sq)::PER;
@@ -309,6 +325,14 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
             };
             if (cpartial) elementwise(std::true_type{});
             else elementwise(std::false_type{});
+            if (WRITE_DS) {
+#pragma unroll
+                for (int g4 = 0; g4 < 4; ++g4) {
+                    const bf16x8 f = dsf[g4 >> 1];
+                    const bf16x4 q4 = (g4 & 1) ? __builtin_shufflevector(f, f, 4, 5, 6, 7) : __builtin_shufflevector(f, f, 0, 1, 2, 3);
+                    *(bf16x4*)(ds_out + 32 * mb + 8 * g4) = q4;
+                }
+            }
             // dV^T += dO^T P and dK^T += Q^T dS  (accumulators stay in AGPRs)
             trfrag_gemm<D, 2, kBPipe, true>(lds_addr(Gs) + tbase + roff, pf, dvacc);
             trfrag_gemm<D, 2, kBPipe, true>(lds_addr(Qs) + tbase + roff, dsf, dkacc);
@@ -329,14 +353,14 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
 
 // One workgroup per work item, or -- with work queues in the tile map -- one per compute unit, pulling
 // items until none is left (see WorkQueue).
-template <int D, bool HAS_DOC>
+template <int D, bool HAS_DOC, bool WRITE_DS>
 __global__ __launch_bounds__(kBwdThreads, D <= 128 ? MA_DKV_WAVES : 1) void attn_bwd_dkv_bf16_kernel(AttnArgs a) {
     extern __shared__ __align__(16) char smem_raw[];
     MA_LDS int* box = (MA_LDS int*)((lds_ptr)smem_raw + (4 * Tile<D>::bytes(kStep) + 2 * kStep * (4 + 4 + 8)));
     WorkQueue wq;
     wq.init(a.map.work_counters, kQueueDkv, work_grid(a.B * a.T, a.Hkv, 1));
     for (int id = wq.next(box); id >= 0; id = wq.next(box)) {
-        attn_bwd_dkv_bf16_item<D, HAS_DOC>(fresh_args(), id);
+        attn_bwd_dkv_bf16_item<D, HAS_DOC, WRITE_DS>(fresh_args(), id);
         __syncthreads();  // the item's LDS (and the box) are free again
     }
     wq.leave();
@@ -593,6 +617,117 @@ __global__ __launch_bounds__(kBwdThreads, D <= 128 ? 2 : 1) void attn_bwd_dq_bf1
     attn_bwd_dq_bf16_item<D, HAS_DOC>(fresh_args(), (int)blockIdx.x);
 }
 
+// ------------------------------------------------------------------------------------------------
+// dQ from the dS^T that the dK/dV kernel left in a.ds
+// ------------------------------------------------------------------------------------------------
+// dQ^T += K^T dS^T and nothing else: no Q / dO / O fragments, no scores, no exponentials.  Per step
+// of 64 kv rows the workgroup stages the K tile and the [64 kv][128 q] slab of dS^T of its q tile;
+// both MFMA operands come from LDS through transposed reads of the same kv rows, so their
+// contraction orders agree by construction.  Every block this kernel reads has been written: it
+// walks the same tile lists as the dK/dV kernel, that kernel writes all blocks of every step it
+// walks, and a block that can hold a visible pair lies inside a step with a visible pair.
+template <int D, bool HAS_DOC>
+__device__ __forceinline__ void attn_bwd_dq_ds_bf16_item(KernArgs& a, const int wg_id) {
+    using TL = Tile<D>;
+    using TS = Tile<kTile>;
+    constexpr int DB = D / 32;
+    constexpr int BN = kStep;
+    constexpr int NW = kBwdThreads / 64;
+    extern __shared__ __align__(16) char smem_raw[];
+    const lds_ptr lds0 = (lds_ptr)smem_raw;
+    auto Kbuf = [&](int i) { return lds0 + i * TL::bytes(BN); };
+    auto Sbuf = [&](int i) { return lds0 + 2 * TL::bytes(BN) + i * TS::bytes(BN); };
+
+    const int tid = fresh_tid(), lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    int i, h, b;
+    if (!map_work(wg_id, a.B * a.T, a.T, a.Hkv, a.Hq / a.Hkv, a.map.q_tile_order, i, h, b)) return;
+    const int tbase = TL::tr_base(lane), sbase = TS::tr_base(lane);
+    const int hk = h / (a.Hq / a.Hkv);
+    const int qw_lo = i * kTile + 32 * w, qw_hi = qw_lo + 31;
+    const bool bounded = a.causal || a.window >= 0;
+    const __bf16* kp = (const __bf16*)a.k.ptr + b * a.k.stride_b + hk * a.k.stride_h;
+    const __bf16* sp = (const __bf16*)a.ds + (((size_t)b * a.Hq + h) * a.T + i) * a.T * (kTile * kTile);   // kv tile 0 of this q tile
+    const int wlim = a.window >= 0 ? (int)min(a.window, (int64_t)0x3fffffff) : 0x7fffffff;
+
+    const size_t mrow = (size_t)b * a.T + i;
+    const bool windowed = a.window >= 0;
+    int blk_lo, blk_hi;
+    visibility_limits(false, qw_lo, qw_hi, 32, bounded, wlim, windowed, blk_lo, blk_hi);
+    const bool use_rng = HAS_DOC && a.map.block_doc_range != nullptr;
+    const int64_t* rng_row = use_rng ? a.map.block_doc_range + (size_t)b * (2 * ((a.S + 63) / 64)) * 2 : nullptr;
+    DocRange own;
+    if (use_rng) {  // (load and wait stay adjacent: the registers of a scalar load in flight must not be touched)
+        own.load(rng_row + (size_t)(min(qw_lo, a.S - 1) / MA_DOC_BLOCK) * 2);
+        own.ready();
+    }
+    StepTable<BN> st;
+    {
+        int lo, hi;
+        visibility_limits(false, i * kTile, i * kTile + kTile - 1, BN, bounded, wlim, windowed, lo, hi);
+        int n_partial, n_full;
+        scalar_load2(a.map.kv_num_blocks + mrow, a.map.full_kv_num_blocks + mrow, n_partial, n_full);
+        st.init(a.map.kv_indices + mrow * a.T, n_partial, a.map.full_kv_indices + mrow * a.T, n_full, 1, false, a.S, lo, hi,
+                blk_lo, blk_hi, rng_row, use_rng ? own.lo() : 0, use_rng ? own.hi() : 0,
+                (MA_LDS uint32_t*)(lds0 + 2 * TL::bytes(BN) + 2 * TS::bytes(BN) + 16) + w * 64);
+        st.prime();
+    }
+
+    f32x16 acc[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[db][v] = 0.f;
+
+    DirectStager<D, BN, NW> sk;
+    DirectStager<kTile, BN, NW> ss;
+    sk.init(w, lane);
+    ss.init(w, lane);
+    const uint32_t ksb = (uint32_t)(a.k.stride_s * 2);
+    auto issue = [&](int buf) {  // K rows r0 .. r0+63 and the matching 64 rows of dS^T (row r0 of the tile list = kv row)
+        sk.issue((const __bf16*)((const char*)kp + (uint64_t)(uint32_t)st.r0 * ksb), Kbuf(buf), w, lane, min(BN, a.S - st.r0), a.k.stride_s);
+        ss.issue(sp + (size_t)st.r0 * kTile, Sbuf(buf), w, lane, BN, kTile);     // slot jt, row r0 % 128: (r0 / 128) * 16384 + (r0 % 128) * 128
+    };
+    bool have = st.next();
+    bool act0 = st.act0, act1 = st.act1;
+    if (have) issue(0);
+
+    for (int n = 0; have; ++n) {
+        const int cur = n & 1;
+        const lds_ptr Ks = Kbuf(cur), Ss = Sbuf(cur);
+        wait_vmem();
+        __syncthreads();
+        const bool skip[BN / 32] = {!act0, !act1};
+        have = st.next();
+        if (have) {
+            act0 = st.act0;
+            act1 = st.act1;
+            issue(cur ^ 1);
+        }
+#pragma unroll 1
+        for (int nb = 0; nb < BN / 32; ++nb) {
+            if (nb ? skip[1] : skip[0]) continue;
+            bf16x8 dsf[2];
+#pragma unroll
+            for (int jj = 0; jj < 2; ++jj) dsf[jj] = TS::tr_frag(Ss, sbase, 32 * nb + 16 * jj, 32 * w);
+            trfrag_gemm<D, 2, kBPipe, true>(lds_addr(Ks) + tbase + (uint32_t)(32 * nb * TL::kPitch), dsf, acc);
+        }
+    }
+
+    __syncthreads();
+    mfma_fence();
+    {
+        constexpr int kPitchO = D * 2 + 16;
+        __bf16* ob = (__bf16*)a.dq.ptr + b * a.dq.stride_b + h * a.dq.stride_h;
+        store_tile_T<D>(lds0 + w * 32 * kPitchO, acc, a.scale, ob, a.dq.stride_s, qw_lo, a.S, lane);
+    }
+}
+
+template <int D, bool HAS_DOC>
+__global__ __launch_bounds__(kBwdThreads, D <= 128 ? 2 : 1) void attn_bwd_dq_ds_bf16_kernel(AttnArgs a) {
+    attn_bwd_dq_ds_bf16_item<D, HAS_DOC>(fresh_args(), (int)blockIdx.x);
+}
+
 template <typename K>
 static int opt_in_lds(K kernel, size_t bytes, const char* name) {
     if (bytes <= 64 * 1024) return MA_OK;
@@ -606,11 +741,36 @@ static int bwd_dd(const AttnArgs& a, hipStream_t st) {
     constexpr int RPB = 256 / (D / 8);
     const int64_t nrows = (int64_t)a.B * a.Hq * a.S;
     int rc = MA_OK;
-    // delta on its own only when the dQ stage, which computes it for its own rows, is not asked for
-    if ((a.stages & MA_BWD_DELTA) && !(a.stages & MA_BWD_DQ)) {
+    const bool hand_over = a.ds != nullptr;  // dS^T goes from the dK/dV kernel to the dQ kernel through a.ds
+    // delta on its own when the dQ stage, which computes it for its own rows, is not asked for, and
+    // always with the hand-over (its dQ kernel reads neither O nor dO)
+    if ((a.stages & MA_BWD_DELTA) && (hand_over || !(a.stages & MA_BWD_DQ))) {
         hipLaunchKernelGGL(attn_delta_bf16_kernel<D>, dim3((unsigned)((nrows + RPB - 1) / RPB)), dim3(256), 0, st, a);
         rc = check_launch("attn_delta_bf16_kernel");
         if (rc) return rc;
+    }
+    const size_t lds_kv = (size_t)4 * Tile<D>::bytes(kStep) + 2 * kStep * (4 + 4 + 8) + 16 + (kBwdThreads / 64) * 256;  // + work-queue box, step tables
+    if (hand_over) {
+        if (a.stages & MA_BWD_DKV) {
+            rc = opt_in_lds(attn_bwd_dkv_bf16_kernel<D, HAS_DOC, true>, lds_kv, "attn_bwd_dkv_bf16");
+            if (rc) return rc;
+            static const int resident = resident_workgroups(attn_bwd_dkv_bf16_kernel<D, HAS_DOC, true>, kBwdThreads, lds_kv);
+            hipLaunchKernelGGL((attn_bwd_dkv_bf16_kernel<D, HAS_DOC, true>), dim3(queue_grid(work_grid(a.B * a.T, a.Hkv, 1), a.map.work_counters, resident), 1, 1),
+                               dim3(kBwdThreads), lds_kv, st, a);
+            rc = check_launch("attn_bwd_dkv_bf16_kernel");
+            if (rc) return rc;
+        }
+        if (a.stages & MA_BWD_DQ) {
+            const size_t lds_q = (size_t)2 * Tile<D>::bytes(kStep) + 2 * Tile<kTile>::bytes(kStep) + 16 + (kBwdThreads / 64) * 256;
+            const size_t lds_store = (size_t)(kBwdThreads / 64) * 32 * (D * 2 + 16);   // the epilogue's scratch
+            const size_t lds = lds_q > lds_store ? lds_q : lds_store;
+            rc = opt_in_lds(attn_bwd_dq_ds_bf16_kernel<D, HAS_DOC>, lds, "attn_bwd_dq_ds_bf16");
+            if (rc) return rc;
+            hipLaunchKernelGGL((attn_bwd_dq_ds_bf16_kernel<D, HAS_DOC>), dim3(work_grid(a.B * a.T, a.Hkv, a.Hq / a.Hkv), 1, 1), dim3(kBwdThreads),
+                               lds, st, a);
+            rc = check_launch("attn_bwd_dq_ds_bf16_kernel");
+        }
+        return rc;
     }
     if (a.stages & MA_BWD_DQ) {  // first: the dK/dV kernel reads the delta this one may be writing
         const size_t lds_q = (size_t)4 * Tile<D>::bytes(kStep) + 2 * kStep * 8 + 16 + (kBwdThreads / 64) * 256;  // K/V ring, kv document ids, step tables
@@ -622,11 +782,10 @@ static int bwd_dd(const AttnArgs& a, hipStream_t st) {
         if (rc) return rc;
     }
     if (a.stages & MA_BWD_DKV) {
-        const size_t lds_kv = (size_t)4 * Tile<D>::bytes(kStep) + 2 * kStep * (4 + 4 + 8) + 16 + (kBwdThreads / 64) * 256;  // + work-queue box, step tables
-        rc = opt_in_lds(attn_bwd_dkv_bf16_kernel<D, HAS_DOC>, lds_kv, "attn_bwd_dkv_bf16");
+        rc = opt_in_lds(attn_bwd_dkv_bf16_kernel<D, HAS_DOC, false>, lds_kv, "attn_bwd_dkv_bf16");
         if (rc) return rc;
-        static const int resident = resident_workgroups(attn_bwd_dkv_bf16_kernel<D, HAS_DOC>, kBwdThreads, lds_kv);
-        hipLaunchKernelGGL((attn_bwd_dkv_bf16_kernel<D, HAS_DOC>), dim3(queue_grid(work_grid(a.B * a.T, a.Hkv, 1), a.map.work_counters, resident), 1, 1), dim3(kBwdThreads), lds_kv,
+        static const int resident = resident_workgroups(attn_bwd_dkv_bf16_kernel<D, HAS_DOC, false>, kBwdThreads, lds_kv);
+        hipLaunchKernelGGL((attn_bwd_dkv_bf16_kernel<D, HAS_DOC, false>), dim3(queue_grid(work_grid(a.B * a.T, a.Hkv, 1), a.map.work_counters, resident), 1, 1), dim3(kBwdThreads), lds_kv,
                            st, a);
         rc = check_launch("attn_bwd_dkv_bf16_kernel");
     }

@@ -68,6 +68,9 @@ struct AttnArgs {
     float scale;
     int B, S, Hq, Hkv, D, T;
     int stages;  // MA_BWD_* mask (backward only)
+    // dS^T handed from the dK/dV kernel to the dQ kernel (backward only, may be NULL): bf16
+    // [B, Hq, T, T, 128 kv, 128 q], one 32 KB slot per (q tile, kv tile) whether visited or not
+    void* ds;
 };
 
 // The argument block as the per-item functions of the queue-driven kernels see it: in the constant

@@ -9,7 +9,7 @@ import torch
 
 from conftest import max_abs, rel_l2
 from maester_amd import build_tile_map, doc_masked_attention, packed_doc_attention, workloads
-from maester_amd.attention import attention_backward, attention_forward
+from maester_amd.attention import attention_backward, attention_forward, backward_workspace_bytes
 from oracle import attention as A
 from oracle import prologue as P
 
@@ -202,6 +202,55 @@ def test_full_size_properties_and_slice(gpu, name):
     starts = (wl.position_ids == 0)
     for h in (0, sp.Hq - 1):
         assert torch.equal(out[:, :, h][starts], wl.xv[:, :, h // G][starts])
+
+
+def _backward_both_ways(gpu, q, k, v, do, ids, scale, window):
+    """(dq, dk, dv) with dS handed from the dK/dV kernel to the dQ kernel through a workspace that starts out full of
+    NaNs (every block the dQ kernel reads must have been written by the dK/dV kernel), and with the dQ kernel
+    recomputing S and dP."""
+    B, S, Hq, D = q.shape
+    Hkv = k.shape[2]
+    tm = build_tile_map(ids, B, S, True, window, device=gpu)
+    out, lse = attention_forward(q, k, v, tm, ids, scale, True, window)
+    ws = torch.full((backward_workspace_bytes(B, S, Hq, Hkv, D, q.dtype, True),), 0xFF, dtype=torch.uint8, device=gpu)
+    bufs = (torch.empty_like(q), torch.empty_like(k), torch.empty_like(v), ws)
+    handed = attention_backward(q, k, v, out, do, lse, tm, ids, scale, True, window, buffers=bufs)
+    handed = tuple(t.clone() for t in handed)
+    again = attention_backward(q, k, v, out, do, lse, tm, ids, scale, True, window, buffers=bufs)
+    assert all(torch.equal(x, y) for x, y in zip(handed, again))
+    recomputed = attention_backward(q, k, v, out, do, lse, tm, ids, scale, True, window, hand_over=False)
+    return handed, recomputed
+
+
+@pytest.mark.parametrize("case", BF16_CASES, ids=[c[0] for c in BF16_CASES])
+def test_bf16_backward_ds_hand_over_and_recompute(gpu, case):
+    _, B, S, Hq, Hkv, D, window, kind = case
+    q, k, v, do = _qkv(B, S, Hq, Hkv, D, torch.bfloat16, 17)
+    ids = _ids(B, S, 18, kind)
+    scale = D ** -0.5
+    _, dq, dk, dv = A.dense_attention_fwd_bwd(q, k, v, do, ids, scale, True, window)
+    gids = None if ids is None else ids.to(gpu)
+    handed, recomputed = _backward_both_ways(gpu, q.to(gpu), k.to(gpu), v.to(gpu), do.to(gpu), gids, scale, window)
+    for got in (handed, recomputed):
+        assert all(bool(torch.isfinite(t).all()) for t in got)
+        for name, a, b in zip(("dq", "dk", "dv"), got, (dq, dk, dv)):
+            _check(a, b, torch.bfloat16, (case[0], name))
+    # the dK/dV kernel computes the same thing either way; delta comes from another kernel (another summation order)
+    assert torch.equal(handed[2], recomputed[2])
+    assert rel_l2(handed[1].float(), recomputed[1].float()) <= 2e-3
+
+
+@pytest.mark.parametrize("name", ["c2", "c3", "c5"])
+def test_full_size_ds_hand_over_reads_only_what_was_written(gpu, name):
+    wl = workloads.make(name).to(gpu)
+    sp = wl.spec
+    handed, recomputed = _backward_both_ways(gpu, wl.xq, wl.xk, wl.xv, wl.dout, wl.document_ids, wl.scale, sp.window)
+    assert all(bool(torch.isfinite(t).all()) for t in handed)
+    assert torch.equal(handed[2], recomputed[2])
+    assert rel_l2(handed[1].float(), recomputed[1].float()) <= 2e-3
+    # both dQ kernels multiply a bf16 dS with K; they differ by the rounding of dS only where the two kernels'
+    # fp32 sums of S and dP differ in the last bits
+    assert rel_l2(handed[0].float(), recomputed[0].float()) <= 2e-3
 
 
 @pytest.mark.parametrize("name", ["c2", "c3", "c4", "c5"])
