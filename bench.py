@@ -291,7 +291,8 @@ def main():
         ("attn_fwd_pair_bf16_kernel" if (sp.Hq // sp.Hkv) % 2 == 0 and sp.D >= 256 and sp.dtype == torch.bfloat16 else "attn_fwd_bf16_kernel"):
             {"ms": t_fwd, "algorithmic_flops": 4 * base},
         "attn_bwd_dkv_bf16_kernel": {"ms": t_dkv, "algorithmic_flops": 6 * base},   # dP, dV, dK
-        ("attn_bwd_dq_ds_bf16_kernel" if has_bwd and hand_over else "attn_bwd_dq_bf16_kernel"):
+        (("attn_bwd_dq_ds_pair_bf16_kernel" if (sp.Hq // sp.Hkv) % 2 == 0 else "attn_bwd_dq_ds_bf16_kernel")
+         if has_bwd and hand_over else "attn_bwd_dq_bf16_kernel"):
             {"ms": t_dq, "algorithmic_flops": 2 * base},                            # dQ
     }
     for v in kern.values():
@@ -318,7 +319,7 @@ def main():
         "dtype": "bf16" if sp.dtype == torch.bfloat16 else "f32", "data": "synthetic",
         "config": {"workload": sp.name, "description": sp.description, "B": sp.B, "S": sp.S, "Hq": sp.Hq,
                    "Hkv": sp.Hkv, "D": sp.D, "window": sp.window, "n_pairs": wl.n_pairs,
-                   "timed_region": "ma_attn_fwd + ma_attn_bwd (delta, dK/dV, dQ) per step, inputs resident in HBM"},
+                   "timed_region": "ma_attn_fwd + ma_attn_bwd (delta, dK/dV with dS hand-over, dQ) per step, inputs resident in HBM"},
         "pct_of_bf16_dense_peak": 100.0 * value / PEAK_BF16_DENSE_TFLOPS,
         "peak_bf16_dense_tflops": PEAK_BF16_DENSE_TFLOPS, "peak_hbm_gbps": PEAK_HBM_GBPS,
         "device": props.name, "gcn_arch": getattr(props, "gcnArchName", ""), "cus": props.multi_processor_count,

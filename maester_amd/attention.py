@@ -133,7 +133,7 @@ def attention_forward(q, k, v, tile_map: TileMap, document_ids, scale, causal=Tr
 
 # Largest workspace the backward takes for handing dS from the dK/dV kernel to the dQ kernel (bytes);
 # above it (long sequences: the slots grow with (S/128)^2) the dQ kernel recomputes S and dP instead.
-DS_WORKSPACE_LIMIT = 24 << 30
+DS_WORKSPACE_LIMIT = 64 << 30
 
 
 def backward_workspace_bytes(B, S, Hq, Hkv, D, dtype, hand_over=None) -> int:

@@ -213,12 +213,15 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
         issue_g(0);
         issue_rows();
     }
-    // where this lane's 4 x 4 values of a 32 x 32 block go: slot (b, head, q tile, kv tile j) of a.ds,
-    // row = the lane's kv row, columns q0 % 128 + 32*mb + 8*g4 + 4*hh .. +3
-    auto ds_row = [&](int head, int q_first) {
-        const size_t slot = (((size_t)b * a.Hq + head) * a.T + (q_first >> 7)) * a.T + j;
-        return (__bf16*)a.ds + slot * (kTile * kTile) + (size_t)(32 * w + r) * kTile + (q_first & (kTile - 1)) + 4 * hh;
+    // Where the dS^T of a step goes: slot (b, head, q tile, kv tile j) of a.ds and, inside it, the half
+    // of the q tile the step covers -- a uniform address, formed on the scalar side; the lane adds the
+    // byte offset of its kv row and of its 8 columns, the block and the column pair are immediates.
+    auto ds_step = [&](int head, int q_first) {
+        const uint32_t slot = (((uint32_t)b * a.Hq + head) * a.T + (q_first >> 7)) * a.T + j;
+        return (char*)a.ds + (uint64_t)__builtin_amdgcn_readfirstlane(slot) * (kTile * kTile * 2) +
+               (uint32_t)__builtin_amdgcn_readfirstlane((q_first & (kTile - 1)) * 2);
     };
+    const uint32_t ds_lane = (uint32_t)((32 * w + r) * (kTile * 2) + 16 * hh);
 
     for (int n = 0; have; ++n) {
         const int cur = n & 1;
@@ -237,7 +240,7 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
         const int cq0 = q0;
         const bool cpartial = partial;
         const bool skip[BM / 32] = {!act0, !act1};  // blocks in which this wave has nothing to do
-        __bf16* ds_out = WRITE_DS ? ds_row(hk * G + rep, cq0) : nullptr;
+        char* ds_out = WRITE_DS ? ds_step(hk * G + rep, cq0) : nullptr;
         have = st.next();
         // The tile loads of the next step are spread over this step's first MFMA chains, one run
         // every few MFMAs (Q tile in the first 32-row block, dO tile in the second): issued in one
@@ -267,7 +270,7 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
             if (mb ? skip[1] : skip[0]) {
                 if (WRITE_DS) {
 #pragma unroll
-                    for (int g4 = 0; g4 < 4; ++g4) *(uint2*)(ds_out + 32 * mb + 8 * g4) = make_uint2(0, 0);
+                    for (int pr = 0; pr < 2; ++pr) *(u32x4*)(ds_out + ds_lane + 64 * mb + 32 * pr) = u32x4{0, 0, 0, 0};
                 }
                 continue;
             }
@@ -326,11 +329,16 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
             if (cpartial) elementwise(std::true_type{});
             else elementwise(std::false_type{});
             if (WRITE_DS) {
+                // A lane holds q columns 8*g4 + 4*hh .. +3 of its kv row; swapping the second half of the
+                // hh = 0 lanes with the first half of the hh = 1 lanes gives every lane 8 consecutive
+                // columns (16*pair + 8*hh .. +7): one 16-byte store per pair instead of two of 8 bytes, and
+                // the two lanes of a row write 32 adjacent bytes.
 #pragma unroll
-                for (int g4 = 0; g4 < 4; ++g4) {
-                    const bf16x8 f = dsf[g4 >> 1];
-                    const bf16x4 q4 = (g4 & 1) ? __builtin_shufflevector(f, f, 4, 5, 6, 7) : __builtin_shufflevector(f, f, 0, 1, 2, 3);
-                    *(bf16x4*)(ds_out + 32 * mb + 8 * g4) = q4;
+                for (int pr = 0; pr < 2; ++pr) {
+                    const u32x4 f = __builtin_bit_cast(u32x4, dsf[pr]);   // dwords 0,1: g4 = 2*pr, dwords 2,3: g4 = 2*pr + 1
+                    const auto s0 = __builtin_amdgcn_permlane32_swap(f[0], f[2], false, false);
+                    const auto s1 = __builtin_amdgcn_permlane32_swap(f[1], f[3], false, false);
+                    *(u32x4*)(ds_out + ds_lane + 64 * mb + 32 * pr) = u32x4{s0[0], s1[0], s0[1], s1[1]};
                 }
             }
             // dV^T += dO^T P and dK^T += Q^T dS  (accumulators stay in AGPRs)
@@ -620,6 +628,9 @@ __global__ __launch_bounds__(kBwdThreads, D <= 128 ? 2 : 1) void attn_bwd_dq_bf1
 // ------------------------------------------------------------------------------------------------
 // dQ from the dS^T that the dK/dV kernel left in a.ds
 // ------------------------------------------------------------------------------------------------
+#ifndef MA_DQ_PAIR_MIN_D
+#define MA_DQ_PAIR_MIN_D 64   // head dims from which an even GQA group goes through the two-head kernel
+#endif
 // dQ^T += K^T dS^T and nothing else: no Q / dO / O fragments, no scores, no exponentials.  Per step
 // of 64 kv rows the workgroup stages the K tile and the [64 kv][128 q] slab of dS^T of its q tile;
 // both MFMA operands come from LDS through transposed reads of the same kv rows, so their
@@ -728,6 +739,148 @@ __global__ __launch_bounds__(kBwdThreads, D <= 128 ? 2 : 1) void attn_bwd_dq_ds_
     attn_bwd_dq_ds_bf16_item<D, HAS_DOC>(fresh_args(), (int)blockIdx.x);
 }
 
+// Two query heads of one kv head per workgroup: the K tile is staged once and every transposed K
+// fragment read from LDS feeds two MFMAs (one per head's dS^T), which halves the kernel's K traffic
+// and LDS reads per FLOP.  The tile loads of the next step are spread over this step's chains: the K
+// tile over the first 32-row block, the two dS^T slabs over the second.
+template <int D, bool HAS_DOC>
+__device__ __forceinline__ void attn_bwd_dq_ds_pair_bf16_item(KernArgs& a, const int wg_id) {
+    using TL = Tile<D>;
+    using TS = Tile<kTile>;
+    constexpr int DB = D / 32;
+    constexpr int BN = kStep;
+    constexpr int NW = kBwdThreads / 64;
+    constexpr int kStage = TL::bytes(BN) + 2 * TS::bytes(BN);      // K tile, dS^T of head 0, dS^T of head 1
+    extern __shared__ __align__(16) char smem_raw[];
+    const lds_ptr lds0 = (lds_ptr)smem_raw;
+    auto Kbuf = [&](int i) { return lds0 + i * kStage; };
+    auto Sbuf = [&](int i, int head) { return lds0 + i * kStage + TL::bytes(BN) + head * TS::bytes(BN); };
+
+    const int tid = fresh_tid(), lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int G = a.Hq / a.Hkv, GP = G / 2;
+    int i, hp, b;
+    if (!map_work(wg_id, a.B * a.T, a.T, a.Hkv, GP, a.map.q_tile_order, i, hp, b)) return;
+    const int hk = hp / GP;
+    const int h0 = hk * G + 2 * (hp % GP);  // the pair is (h0, h0 + 1)
+    const int tbase = TL::tr_base(lane), sbase = TS::tr_base(lane);
+    const int qw_lo = i * kTile + 32 * w, qw_hi = qw_lo + 31;
+    const bool bounded = a.causal || a.window >= 0;
+    const __bf16* kp = (const __bf16*)a.k.ptr + b * a.k.stride_b + hk * a.k.stride_h;
+    const size_t head_slots = (size_t)a.T * a.T * (kTile * kTile);
+    const __bf16* sp0 = (const __bf16*)a.ds + (((size_t)b * a.Hq + h0) * a.T + i) * a.T * (kTile * kTile);
+    const __bf16* sp1 = sp0 + head_slots;
+    const int wlim = a.window >= 0 ? (int)min(a.window, (int64_t)0x3fffffff) : 0x7fffffff;
+
+    const size_t mrow = (size_t)b * a.T + i;
+    const bool windowed = a.window >= 0;
+    int blk_lo, blk_hi;
+    visibility_limits(false, qw_lo, qw_hi, 32, bounded, wlim, windowed, blk_lo, blk_hi);
+    const bool use_rng = HAS_DOC && a.map.block_doc_range != nullptr;
+    const int64_t* rng_row = use_rng ? a.map.block_doc_range + (size_t)b * (2 * ((a.S + 63) / 64)) * 2 : nullptr;
+    DocRange own;
+    if (use_rng) {  // (load and wait stay adjacent: the registers of a scalar load in flight must not be touched)
+        own.load(rng_row + (size_t)(min(qw_lo, a.S - 1) / MA_DOC_BLOCK) * 2);
+        own.ready();
+    }
+    StepTable<BN> st;
+    {
+        int lo, hi;
+        visibility_limits(false, i * kTile, i * kTile + kTile - 1, BN, bounded, wlim, windowed, lo, hi);
+        int n_partial, n_full;
+        scalar_load2(a.map.kv_num_blocks + mrow, a.map.full_kv_num_blocks + mrow, n_partial, n_full);
+        st.init(a.map.kv_indices + mrow * a.T, n_partial, a.map.full_kv_indices + mrow * a.T, n_full, 1, false, a.S, lo, hi,
+                blk_lo, blk_hi, rng_row, use_rng ? own.lo() : 0, use_rng ? own.hi() : 0,
+                (MA_LDS uint32_t*)(lds0 + 2 * kStage + 16) + w * 64);
+        st.prime();
+    }
+
+    f32x16 acc0[DB], acc1[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc0[db][v] = acc1[db][v] = 0.f;
+
+    DirectStager<D, BN, NW> sk;
+    DirectStager<kTile, BN, NW> ss;
+    sk.init(w, lane);
+    ss.init(w, lane);
+    const uint32_t ksb = (uint32_t)(a.k.stride_s * 2);
+    auto issue = [&](int buf) {
+        sk.issue((const __bf16*)((const char*)kp + (uint64_t)(uint32_t)st.r0 * ksb), Kbuf(buf), w, lane, min(BN, a.S - st.r0), a.k.stride_s);
+        ss.issue(sp0 + (size_t)st.r0 * kTile, Sbuf(buf, 0), w, lane, BN, kTile);
+        ss.issue(sp1 + (size_t)st.r0 * kTile, Sbuf(buf, 1), w, lane, BN, kTile);
+    };
+    const int k_runs = decltype(sk)::runs_of(w), s_runs = decltype(ss)::runs_of(w);
+    bool have = st.next();
+    bool act0 = st.act0, act1 = st.act1;
+    if (have) issue(0);
+
+    for (int n = 0; have; ++n) {
+        const int cur = n & 1;
+        wait_vmem();
+        __syncthreads();
+        const bool skip0 = !act0, skip1 = !act1;
+        have = st.next();
+        int pace = 0;
+        const __bf16 *ksrc = kp, *s0src = sp0, *s1src = sp1;
+        if (have) {
+            act0 = st.act0;
+            act1 = st.act1;
+            ksrc = (const __bf16*)((const char*)kp + (uint64_t)(uint32_t)st.r0 * ksb);
+            s0src = sp0 + (size_t)st.r0 * kTile;
+            s1src = sp1 + (size_t)st.r0 * kTile;
+            // (smaller head dims have too few MFMAs per block to hide the runs behind: all at once)
+            constexpr bool kPaced = decltype(sk)::PER <= (2 * 2 * DB) / 3 && 2 * decltype(ss)::PER <= (2 * 2 * DB) / 3;
+            const bool spread = kPaced & (st.r0 + BN <= a.S) & !skip0 & !skip1;
+            pace = __builtin_amdgcn_readfirstlane(spread ? 1 : 0);
+            if (!pace) issue(cur ^ 1);
+        }
+        const uint32_t kdst = lds_addr(Kbuf(cur ^ 1)), s0dst = lds_addr(Sbuf(cur ^ 1, 0)), s1dst = lds_addr(Sbuf(cur ^ 1, 1));
+        const int k_lim = pace ? k_runs : 0, s_lim = pace ? s_runs : 0;
+        constexpr int kEvery = 3;                                   // one run every third MFMA
+
+        static_for<0, BN / 32>([&](auto nb_c) {
+            constexpr int nb = decltype(nb_c)::value;
+            if (nb ? skip1 : skip0) return;
+            bf16x8 dsf0[2], dsf1[2];
+#pragma unroll
+            for (int jj = 0; jj < 2; ++jj) {
+                dsf0[jj] = TS::tr_frag(Sbuf(cur, 0), sbase, 32 * nb + 16 * jj, 32 * w);
+                dsf1[jj] = TS::tr_frag(Sbuf(cur, 1), sbase, 32 * nb + 16 * jj, 32 * w);
+            }
+            auto pace_hook = [&](auto idx) {
+                constexpr int m = decltype(idx)::value;
+                if constexpr (m % kEvery == kEvery - 1) {
+                    constexpr int run = m / kEvery;
+                    if constexpr (nb == 0) {
+                        sk.template issue_one<run>(ksrc, kdst, w, k_lim, ksb);
+                    } else if constexpr (run < decltype(ss)::PER) {
+                        ss.template issue_one<run>(s0src, s0dst, w, s_lim, kTile * 2);
+                    } else {
+                        ss.template issue_one<run - decltype(ss)::PER>(s1src, s1dst, w, s_lim, kTile * 2);
+                    }
+                }
+            };
+            trfrag_gemm_dual<D, 2, kBPipe>(lds_addr(Kbuf(cur)) + tbase + (uint32_t)(32 * nb * TL::kPitch), dsf0, dsf1, acc0, acc1, pace_hook);
+        });
+    }
+
+    __syncthreads();
+    mfma_fence();
+    {
+        constexpr int kPitchO = D * 2 + 16;
+        __bf16* ob = (__bf16*)a.dq.ptr + b * a.dq.stride_b + h0 * a.dq.stride_h;
+        store_tile_T<D>(lds0 + w * 32 * kPitchO, acc0, a.scale, ob, a.dq.stride_s, qw_lo, a.S, lane);
+        store_tile_T<D>(lds0 + w * 32 * kPitchO, acc1, a.scale, ob + a.dq.stride_h, a.dq.stride_s, qw_lo, a.S, lane);
+    }
+}
+
+template <int D, bool HAS_DOC>
+__global__ __launch_bounds__(kBwdThreads, 1) void attn_bwd_dq_ds_pair_bf16_kernel(AttnArgs a) {
+    attn_bwd_dq_ds_pair_bf16_item<D, HAS_DOC>(fresh_args(), (int)blockIdx.x);
+}
+
 template <typename K>
 static int opt_in_lds(K kernel, size_t bytes, const char* name) {
     if (bytes <= 64 * 1024) return MA_OK;
@@ -760,7 +913,15 @@ static int bwd_dd(const AttnArgs& a, hipStream_t st) {
             rc = check_launch("attn_bwd_dkv_bf16_kernel");
             if (rc) return rc;
         }
-        if (a.stages & MA_BWD_DQ) {
+        const int G = a.Hq / a.Hkv;
+        if ((a.stages & MA_BWD_DQ) && G % 2 == 0 && D >= MA_DQ_PAIR_MIN_D) {
+            const size_t lds_q = (size_t)2 * (Tile<D>::bytes(kStep) + 2 * Tile<kTile>::bytes(kStep)) + 16 + (kBwdThreads / 64) * 256;
+            rc = opt_in_lds(attn_bwd_dq_ds_pair_bf16_kernel<D, HAS_DOC>, lds_q, "attn_bwd_dq_ds_pair_bf16");
+            if (rc) return rc;
+            hipLaunchKernelGGL((attn_bwd_dq_ds_pair_bf16_kernel<D, HAS_DOC>), dim3(work_grid(a.B * a.T, a.Hkv, G / 2), 1, 1), dim3(kBwdThreads),
+                               lds_q, st, a);
+            rc = check_launch("attn_bwd_dq_ds_pair_bf16_kernel");
+        } else if (a.stages & MA_BWD_DQ) {
             const size_t lds_q = (size_t)2 * Tile<D>::bytes(kStep) + 2 * Tile<kTile>::bytes(kStep) + 16 + (kBwdThreads / 64) * 256;
             const size_t lds_store = (size_t)(kBwdThreads / 64) * 32 * (D * 2 + 16);   // the epilogue's scratch
             const size_t lds = lds_q > lds_store ? lds_q : lds_store;
