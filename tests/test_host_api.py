@@ -48,6 +48,10 @@ def test_workspace_sizes():
     assert L.ma_tile_map_workspace_bytes(1, 129) == 16 + 2 * 16 + 16 + 4 * 4   # T = 2: 4 class bytes rounded up to 16
     assert L.ma_tile_map_workspace_bytes(0, 10) == 0
     assert L.ma_attn_bwd_workspace_bytes(4, 8192, 8, 4, 256) == 4 * 8 * 8192 * 4
+    # with room for dS: delta (rounded up to 256 bytes) + one 32 KB slot per (batch row, query head, q tile, kv tile)
+    assert L.ma_attn_bwd_ds_workspace_bytes(4, 8192, 8, 4, 256) == 4 * 8 * 8192 * 4 + 4 * 8 * 64 * 64 * 32768
+    assert L.ma_attn_bwd_ds_workspace_bytes(1, 130, 2, 1, 64) == 1280 + 2 * 2 * 2 * 32768     # 1040 bytes of delta -> 1280
+    assert L.ma_attn_bwd_ds_workspace_bytes(0, 8192, 8, 4, 256) == 0
     assert L.ma_prologue_bwd_workspace_bytes(4, 8192, 8, 4, 256) > 0
 
 
@@ -202,3 +206,17 @@ def test_tile_map_struct_matches_the_header():
     assert fields == [n for n, _ in MaTileMap._fields_] and len(fields) == 12
     assert int(re.search(r"#define MA_WORK_COUNTERS (\d+)", hdr).group(1)) == _lib.MA_WORK_COUNTERS
     assert int(re.search(r"#define MA_DOC_BLOCK (\d+)", hdr).group(1)) == _lib.MA_DOC_BLOCK
+
+
+def test_backward_workspace_choice():
+    import torch
+    from maester_amd import attention as A
+    L = _lib.lib()
+    small, large = L.ma_attn_bwd_workspace_bytes(4, 8192, 8, 4, 256), L.ma_attn_bwd_ds_workspace_bytes(4, 8192, 8, 4, 256)
+    assert A.backward_workspace_bytes(4, 8192, 8, 4, 256, torch.bfloat16) == large          # 4.3 GB: taken
+    assert A.backward_workspace_bytes(4, 8192, 8, 4, 256, torch.float32) == small           # the hand-over is a bf16 path
+    assert A.backward_workspace_bytes(4, 8192, 8, 4, 256, torch.bfloat16, hand_over=False) == small
+    assert A.backward_workspace_bytes(4, 8192, 8, 4, 256, torch.float32, hand_over=True) == small
+    # slots grow with (S / 128)^2: past the limit the dQ kernel recomputes instead
+    assert L.ma_attn_bwd_ds_workspace_bytes(8, 131072, 8, 4, 256) > A.DS_WORKSPACE_LIMIT
+    assert A.backward_workspace_bytes(8, 131072, 8, 4, 256, torch.bfloat16) == L.ma_attn_bwd_workspace_bytes(8, 131072, 8, 4, 256)
