@@ -198,8 +198,10 @@ int ma_attn_fwd(const ma_tensor4* q, const ma_tensor4* k, const ma_tensor4* v, c
  * With ma_attn_bwd_ds_workspace_bytes(...) bytes or more (bf16 only) the dK/dV kernel, which forms
  * dS anyway, also leaves it in the workspace (bf16, one 32 KB slot per pair of tiles and query
  * head, B*Hq*T*T slots of which only the visited ones are touched) and the dQ kernel reduces to
- * dQ = scale * dS K instead of recomputing S and dO V^T: same results to the last bit of the
- * bf16 dS, fewer MFMAs, for workspace that grows with T^2 (4.3 GB at B=4, S=8192, Hq=8). */
+ * dQ = scale * dS K instead of recomputing S and dO V^T: the same dK and dV up to the summation
+ * order of delta, the same dQ up to the rounding of dS to bf16 (which both variants do before the
+ * product), fewer MFMAs, for a workspace that grows with T^2 (4.3 GB at B=4, S=8192, Hq=8).
+ * Nothing in the workspace needs initialising. */
 size_t ma_attn_bwd_workspace_bytes(int B, int S, int Hq, int Hkv, int D);
 size_t ma_attn_bwd_ds_workspace_bytes(int B, int S, int Hq, int Hkv, int D);
 int ma_attn_bwd(const ma_tensor4* q, const ma_tensor4* k, const ma_tensor4* v, const ma_tensor4* out,
