@@ -13,7 +13,7 @@ from .attention import (PackedDocAttention, packed_doc_attention, qk_norm_rope, 
 from .gemma_attention import GemmaAttention, GemmaAttentionConfig
 from .rmsnorm import RMSNorm, rms_norm
 from .linear_ce import ce_rows, linear_cross_entropy
-from .gemma_layers import GemmaLayerConfig, GemmaMLP, Gemma2DecoderLayer, GemmaModel
+from .gemma_layers import GemmaLayerConfig, GemmaMLP, Gemma2DecoderLayer, GemmaModel, GemmaTextModel
 from .packed_ids import (generate_position_ids, generate_document_ids, packed_collate_ids, boundaries_to_tensors,
                          device_packed_ids)
 
@@ -21,5 +21,5 @@ __all__ = [
     "TileMap", "build_tile_map", "precompute_rope_tables", "PackedDocAttention", "packed_doc_attention",
     "qk_norm_rope", "doc_masked_attention", "GemmaAttention", "GemmaAttentionConfig",
     "generate_position_ids", "generate_document_ids", "packed_collate_ids", "boundaries_to_tensors",
-    "device_packed_ids", "RMSNorm", "rms_norm", "ce_rows", "linear_cross_entropy", "GemmaLayerConfig", "GemmaMLP", "Gemma2DecoderLayer", "GemmaModel",
+    "device_packed_ids", "RMSNorm", "rms_norm", "ce_rows", "linear_cross_entropy", "GemmaLayerConfig", "GemmaMLP", "Gemma2DecoderLayer", "GemmaModel", "GemmaTextModel",
 ]

@@ -6,6 +6,9 @@ Counterparts of ``GemmaMLP`` (maester/models/gemma/model.py:177-199), ``Gemma2De
 ids of a step are built once (``build_step_inputs``) and handed to every layer; local and global
 layers alternate as ``attn_types`` says; the four sandwich norms run as fused kernels, the two
 post-norms with their residual add folded in.  The projections and the MLP stay torch GEMMs.
+``GemmaTextModel`` puts the token embedding in front and the tied-embedding loss behind
+(model.py:570-769): ``forward(tokens, labels, position_ids, document_ids)`` returns the loss of the
+fused linear + cross-entropy, or the logits without labels.
 """
 from __future__ import annotations
 
@@ -16,6 +19,7 @@ import torch.nn.functional as F
 from torch import nn
 
 from .gemma_attention import GemmaAttention, GemmaAttentionConfig, StepInputs, build_step_inputs
+from .linear_ce import linear_cross_entropy
 from .rmsnorm import RMSNorm
 
 
@@ -28,6 +32,7 @@ class GemmaLayerConfig(GemmaAttentionConfig):
     attn_types: tuple | None = None          # e.g. ("local_sliding",) * 5 + ("global",)
     use_pre_ffw_norm: bool = True
     use_post_ffw_norm: bool = True
+    vocab_size: int = 0                      # GemmaTextModel only
 
 
 class GemmaMLP(nn.Module):
@@ -103,3 +108,36 @@ class GemmaModel(nn.Module):
         for layer in self.layers:
             layer.init_weights(init_std)
         self.norm.reset_parameters()
+
+
+class GemmaTextModel(nn.Module):
+    """Counterpart of the reference's ``GemmaTextModel`` (model.py:570-769) with the same parameter
+    names (``tok_embeddings.weight``, ``model.layers.*``, ``model.norm.weight``) and the same
+    ``forward(tokens, labels=None, position_ids=None, document_ids=None)``: embeddings scaled by
+    sqrt(dim) (the factor rounded to the activation dtype, as there), the layer stack on one step's
+    tile maps, then the loss against the tied embedding table (``labels`` given, -100 ignored) or the
+    logits."""
+
+    def __init__(self, config: GemmaLayerConfig):
+        super().__init__()
+        if config.vocab_size <= 0:
+            raise ValueError("GemmaTextModel needs config.vocab_size")
+        self.config = config
+        self.model_args = config
+        self.vocab_size = config.vocab_size
+        self.n_layers = config.n_layers
+        self.tok_embeddings = nn.Embedding(config.vocab_size, config.dim)
+        self.model = GemmaModel(config)
+
+    def init_weights(self, init_std: float = 0.02):
+        nn.init.normal_(self.tok_embeddings.weight, std=init_std)
+        self.model.init_weights(init_std)
+
+    def forward(self, tokens: torch.Tensor, labels: torch.Tensor | None = None, position_ids=None, document_ids=None):
+        hidden_states = self.tok_embeddings(tokens)
+        normalizer = torch.tensor(self.config.dim ** 0.5, dtype=hidden_states.dtype, device=hidden_states.device)
+        hidden_states = self.model(hidden_states * normalizer, position_ids, document_ids)
+        weight = self.tok_embeddings.weight
+        if labels is not None:
+            return linear_cross_entropy(hidden_states, weight, labels)
+        return torch.matmul(hidden_states, weight.t())

@@ -117,3 +117,43 @@ def test_layer_stack_shares_the_steps_tile_maps(gpu):
     y.float().pow(2).mean().backward()
     assert all(p.grad is not None and torch.isfinite(p.grad.float()).all() and float(p.grad.float().abs().sum()) > 0
                for p in model.parameters())
+
+
+def test_text_model_tokens_to_loss(gpu):
+    """Tokens in, loss out (counterpart of GemmaTextModel.forward with labels, maester/models/gemma/model.py:654-769):
+    embedding, two layers on one step's tile maps, final norm, fused linear + cross-entropy against the tied
+    embedding table -- against the same computation in fp32 on the CPU with the oracle's pieces."""
+    from maester_amd.gemma_layers import GemmaLayerConfig, GemmaTextModel
+    from oracle import linear_ce as LCE
+    from oracle import prologue as P
+    torch.manual_seed(2)
+    cfg = GemmaLayerConfig(dim=256, n_heads=4, num_key_value_heads=2, head_dim=128, max_seq_len=512, sliding_window_size=64,
+                           intermediate_size=512, n_layers=2, attn_types=("local_sliding", "global"), vocab_size=1000)
+    B, S = 2, 290
+    rows = [[(0, 0, 90), (1, 90, 200)], [(2, 0, 150), (3, 150, 100)]]
+    pos, doc = packed_ids.packed_collate_ids(rows, S)
+    model = GemmaTextModel(cfg).to(gpu).to(torch.bfloat16)
+    model.init_weights(0.06)
+    assert {"tok_embeddings.weight", "model.norm.weight", "model.layers.0.self_attn.qkv_proj.weight"} <= set(model.state_dict())
+    tokens = torch.randint(0, cfg.vocab_size, (B, S))
+    labels = torch.roll(tokens, -1, 1)
+    labels[:, :40] = -100                                      # prompt tokens masked
+    labels[doc < 0] = -100                                     # padding
+    loss = model(tokens.to(gpu), labels.to(gpu), pos.to(gpu), doc.to(gpu))
+    assert loss.shape == () and loss.dtype == torch.float32
+
+    step = build_step_inputs(cfg, B, S, pos.to(gpu), doc.to(gpu))
+    emb = model.tok_embeddings.weight.detach().float().cpu()
+    ref = emb[tokens] * float(torch.tensor(cfg.dim ** 0.5, dtype=torch.bfloat16))
+    for layer, window in zip(model.model.layers, (64, None)):
+        ref = _reference_layer(layer, ref, step, window)
+    ref = P.rms_norm(ref, model.model.norm.weight.detach().float().cpu())
+    want = LCE.linear_cross_entropy(ref.reshape(B * S, -1).numpy(), emb.numpy(), labels.reshape(-1).numpy())["loss"]
+    assert abs(float(loss) - want) <= 2e-2 * max(1.0, abs(want)), (float(loss), want)
+
+    loss.backward()
+    assert all(p.grad is not None and torch.isfinite(p.grad.float()).all() and float(p.grad.float().abs().sum()) > 0
+               for p in model.parameters())
+    # the tied table gets gradient from both of its uses: the rows of tokens that were looked up and, through the loss, all rows
+    logits = model(tokens.to(gpu), None, pos.to(gpu), doc.to(gpu))
+    assert logits.shape == (B, S, cfg.vocab_size)
