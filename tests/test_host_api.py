@@ -220,3 +220,20 @@ def test_backward_workspace_choice():
     # slots grow with (S / 128)^2: past the limit the dQ kernel recomputes instead
     assert L.ma_attn_bwd_ds_workspace_bytes(8, 131072, 8, 4, 256) > A.DS_WORKSPACE_LIMIT
     assert A.backward_workspace_bytes(8, 131072, 8, 4, 256, torch.bfloat16) == L.ma_attn_bwd_workspace_bytes(8, 131072, 8, 4, 256)
+
+
+def test_text_model_mirrors_reference_parameter_names():
+    # maester/models/gemma/model.py:570-585 (tok_embeddings, model), 524-540 (layers, norm), 446-476 (the layer's modules)
+    from maester_amd.gemma_layers import GemmaLayerConfig, GemmaTextModel
+    cfg = GemmaLayerConfig(dim=64, n_heads=2, num_key_value_heads=1, head_dim=64, max_seq_len=128, sliding_window_size=32,
+                           intermediate_size=128, n_layers=2, attn_types=("local_sliding", "global"), vocab_size=100)
+    keys = set(GemmaTextModel(cfg).state_dict())
+    for name in ("tok_embeddings.weight", "model.norm.weight", "model.layers.1.self_attn.qkv_proj.weight",
+                 "model.layers.0.self_attn.o_proj.weight", "model.layers.0.self_attn.query_norm.weight",
+                 "model.layers.0.mlp.gate_proj.weight", "model.layers.0.mlp.up_proj.weight", "model.layers.0.mlp.down_proj.weight",
+                 "model.layers.0.input_layernorm.weight", "model.layers.0.post_attention_layernorm.weight",
+                 "model.layers.0.pre_feedforward_layernorm.weight", "model.layers.0.post_feedforward_layernorm.weight"):
+        assert name in keys, name
+    with pytest.raises(ValueError):
+        GemmaTextModel(GemmaLayerConfig(dim=64, n_heads=2, num_key_value_heads=1, head_dim=64, max_seq_len=128,
+                                        intermediate_size=128))
