@@ -117,12 +117,14 @@ def loss_block(dev, rows, dim, vocab, dtype, with_torch):
     t_all = time_region(lambda: linear_ce_forward(e, c, t), 5, 2)
     step = default_chunk_rows(vocab, e.element_size(), rows)
     blk = torch.mm(e[:step], c.t())
-    de, dc = torch.empty_like(e[:step]), torch.empty_like(c)
+    from maester_amd.linear_ce import transpose
+    de, dc_t = torch.empty_like(e[:step]), torch.empty(dim, vocab, dtype=dtype, device=dev)
+    c_t, e_t = transpose(c), transpose(e[:step].contiguous())
 
-    def gemms():
+    def gemms():       # the three products of a block in the operand orders the loss uses
         torch.mm(e[:step], c.t(), out=blk)
-        torch.mm(blk, c, out=de)
-        torch.mm(blk.t(), e[:step], out=dc)
+        torch.mm(blk, c_t.t(), out=de)
+        torch.mm(e_t, blk, out=dc_t)
     t_gemm = time_region(gemms, 5, 2)
     torch.mm(e[:step], c.t(), out=blk)
     t_rows = time_region(lambda: ce_rows(blk, t[:step]), 10, 3)
@@ -133,7 +135,7 @@ def loss_block(dev, rows, dim, vocab, dtype, with_torch):
            "library_gemms_ms_per_block": t_gemm, "library_gemm_tflops": 6.0 * step * vocab * dim / (t_gemm * 1e-3) / 1e12,
            "ce_rows_kernel": {"ms_per_block": t_rows, "algorithmic_bytes": row_bytes, "gbps": row_bytes / (t_rows * 1e-3) / 1e9,
                               "frac_hbm_peak": row_bytes / (t_rows * 1e-3) / 1e9 / PEAK_HBM_GBPS}}
-    del blk, de, dc
+    del blk, de, dc_t, c_t, e_t
     if with_torch:
         # the reference's materialising path (train.py:258-259) with torch's own kernels on the same inputs
         try:

@@ -138,14 +138,15 @@ int ma_rmsnorm_bwd(const void* x, const float* weight, const float* rstd, const 
  *   soft cap's derivative), zeros for a row that does not count; grad_scale: device fp32 or NULL (= 1).
  * ma_ce_loss_reduce: loss[0] = (sum of nll[0..n) in a fixed order) * scale[0]; scale device fp32 or
  *   NULL (= 1).  With scale = stats + 1 and no row that counts the loss is NaN, as torch's is.
- * ma_transpose: dst[c, r] = src[r, c] for contiguous src [rows, cols], dst [cols, rows] of dtype (the
- *   copy of the classifier that is contiguous along the vocabulary, for the d hidden GEMM);
- *   rows <= 65535 * 64. */
+ * ma_transpose: dst[c, r] = src[r, c] for contiguous src [rows, cols] of src_dtype and dst [cols, rows]
+ *   of dst_dtype: the same dtype (the copy of the classifier that is contiguous along the
+ *   vocabulary, for the d hidden GEMM) or fp32 -> bf16 (the weight gradient, summed over row blocks
+ *   in fp32 as [K, V], handed back as [V, K] in the activation dtype); rows <= 65535 * 64. */
 int ma_ce_valid_count(const int64_t* targets, int64_t n, int64_t ignore_index, int64_t vocab, float* stats, void* stream);
 int ma_ce_rows(void* logits, int64_t pitch, const int64_t* targets, int64_t rows, int64_t vocab, int64_t ignore_index,
                float softcap, const float* grad_scale, float* lse, float* nll, int write_grad, int dtype, void* stream);
 int ma_ce_loss_reduce(const float* nll, int64_t n, const float* scale, float* loss, void* stream);
-int ma_transpose(const void* src, void* dst, int64_t rows, int64_t cols, int dtype, void* stream);
+int ma_transpose(const void* src, void* dst, int64_t rows, int64_t cols, int src_dtype, int dst_dtype, void* stream);
 
 /* ---- fused QK-RMSNorm + RoPE prologue ------------------------------------------------------------
  * Replaces query_norm/key_norm (model.py:135-172, 366-368) followed by apply_rotary_emb

@@ -84,7 +84,7 @@ def lib() -> ctypes.CDLL:
     L.ma_ce_rows.argtypes = [c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64, c_float, c_void_p, c_void_p, c_void_p, c_int,
                              c_int, c_void_p]
     L.ma_transpose.restype = c_int
-    L.ma_transpose.argtypes = [c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p]
+    L.ma_transpose.argtypes = [c_void_p, c_void_p, c_int64, c_int64, c_int, c_int, c_void_p]
     L.ma_ce_loss_reduce.restype = c_int
     L.ma_ce_loss_reduce.argtypes = [c_void_p, c_int64, c_void_p, c_void_p, c_void_p]
     L.ma_rmsnorm_bwd.restype = c_int

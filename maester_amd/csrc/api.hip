@@ -174,13 +174,16 @@ int ma_ce_rows(void* logits, int64_t pitch, const int64_t* targets, int64_t rows
                           dtype, (hipStream_t)stream);
 }
 
-int ma_transpose(const void* src, void* dst, int64_t rows, int64_t cols, int dtype, void* stream) {
+int ma_transpose(const void* src, void* dst, int64_t rows, int64_t cols, int src_dtype, int dst_dtype, void* stream) {
     const char* who = "ma_transpose";
-    MA_TRY(check_dtype(who, dtype));
+    MA_TRY(check_dtype(who, src_dtype));
+    MA_TRY(check_dtype(who, dst_dtype));
+    if (src_dtype == MA_DTYPE_BF16 && dst_dtype != MA_DTYPE_BF16)
+        return fail(MA_ERR_UNSUPPORTED, "%s: bf16 -> fp32 is not offered (same dtype, or fp32 -> bf16)", who);
     if (!src || !dst || src == dst) return fail(MA_ERR_BAD_ARG, "%s: src / dst is NULL, or the same buffer", who);
     if (rows <= 0 || cols <= 0) return fail(MA_ERR_BAD_ARG, "%s: rows=%lld, cols=%lld must be positive", who, (long long)rows, (long long)cols);
     if ((rows + 63) / 64 > 65535) return fail(MA_ERR_UNSUPPORTED, "%s: rows=%lld exceeds 65535 tiles of 64", who, (long long)rows);
-    return launch_transpose(src, dst, rows, cols, dtype, (hipStream_t)stream);
+    return launch_transpose(src, dst, rows, cols, src_dtype, dst_dtype, (hipStream_t)stream);
 }
 
 int ma_ce_loss_reduce(const float* nll, int64_t n, const float* scale, float* loss, void* stream) {

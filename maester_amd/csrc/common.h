@@ -53,7 +53,7 @@ int launch_rmsnorm_bwd(const void* x, const float* weight, const float* rstd, co
                        int64_t rows, int dim, int unit, int dtype, hipStream_t st);
 int launch_ce_rows(void* logits, int64_t pitch, const int64_t* targets, int64_t rows, int vocab, int64_t ignore_index,
                    float softcap, const float* grad_scale, float* lse, float* nll, int write_grad, int dtype, hipStream_t stream);
-int launch_transpose(const void* src, void* dst, int64_t rows, int64_t cols, int dtype, hipStream_t stream);
+int launch_transpose(const void* src, void* dst, int64_t rows, int64_t cols, int src_dtype, int dst_dtype, hipStream_t stream);
 int launch_ce_valid_count(const int64_t* targets, int64_t n, int64_t ignore_index, int vocab, float* stats, hipStream_t stream);
 int launch_ce_loss_reduce(const float* nll, int64_t n, const float* scale, float* loss, hipStream_t stream);
 

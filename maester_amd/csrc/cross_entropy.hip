@@ -240,39 +240,52 @@ __global__ __launch_bounds__(kCeReduceThreads) void ce_loss_reduce_kernel(const 
 // 64 x 64 tiles through LDS, 16-byte accesses on both sides where the shape allows.
 constexpr int kTrTile = 64;
 
-template <typename T>
-__global__ __launch_bounds__(256) void transpose_kernel(const T* __restrict__ src, T* __restrict__ dst, int64_t rows, int64_t cols) {
-    constexpr int V = 16 / sizeof(T);                              // elements per 16-byte access
-    constexpr int kPerRow = kTrTile / V;                           // accesses per tile row
-    __shared__ T tile[kTrTile][kTrTile + 2];
+template <typename TO, typename TI>
+__device__ __forceinline__ TO convert_elem(TI x);
+template <>
+__device__ __forceinline__ uint16_t convert_elem<uint16_t, uint16_t>(uint16_t x) { return x; }
+template <>
+__device__ __forceinline__ float convert_elem<float, float>(float x) { return x; }
+template <>
+__device__ __forceinline__ uint16_t convert_elem<uint16_t, float>(float x) {  // round to nearest even, like torch's cast
+    const __bf16 b = (__bf16)x;
+    return *(const uint16_t*)&b;
+}
+
+// TI -> TO: same type, or fp32 in and bf16 out (the weight gradient summed in fp32, handed back in bf16)
+template <typename TI, typename TO>
+__global__ __launch_bounds__(256) void transpose_kernel(const TI* __restrict__ src, TO* __restrict__ dst, int64_t rows, int64_t cols) {
+    constexpr int VI = 16 / sizeof(TI), VO = 16 / sizeof(TO);      // elements per 16-byte access
+    constexpr int kInPerRow = kTrTile / VI, kOutPerRow = kTrTile / VO;
+    __shared__ TO tile[kTrTile][kTrTile + 2];
     const int64_t r0 = (int64_t)blockIdx.y * kTrTile, c0 = (int64_t)blockIdx.x * kTrTile;
-    const bool vec_in = cols % V == 0 && ((uintptr_t)src & 15) == 0, vec_out = rows % V == 0 && ((uintptr_t)dst & 15) == 0;
-    for (int a = threadIdx.x; a < kTrTile * kPerRow; a += 256) {
-        const int r = a / kPerRow, c = (a % kPerRow) * V;
+    const bool vec_in = cols % VI == 0 && ((uintptr_t)src & 15) == 0, vec_out = rows % VO == 0 && ((uintptr_t)dst & 15) == 0;
+    for (int a = threadIdx.x; a < kTrTile * kInPerRow; a += 256) {
+        const int r = a / kInPerRow, c = (a % kInPerRow) * VI;
         if (r0 + r >= rows) continue;
-        const T* p = src + (r0 + r) * cols + c0 + c;
-        if (vec_in && c0 + c + V <= cols) {
+        const TI* p = src + (r0 + r) * cols + c0 + c;
+        if (vec_in && c0 + c + VI <= cols) {
             const uint4 q = *(const uint4*)p;
-            const T* e = (const T*)&q;
+            const TI* e = (const TI*)&q;
 #pragma unroll
-            for (int i = 0; i < V; ++i) tile[r][c + i] = e[i];
+            for (int i = 0; i < VI; ++i) tile[r][c + i] = convert_elem<TO, TI>(e[i]);
         } else {
-            for (int i = 0; i < V && c0 + c + i < cols; ++i) tile[r][c + i] = p[i];
+            for (int i = 0; i < VI && c0 + c + i < cols; ++i) tile[r][c + i] = convert_elem<TO, TI>(p[i]);
         }
     }
     __syncthreads();
-    for (int a = threadIdx.x; a < kTrTile * kPerRow; a += 256) {
-        const int c = a / kPerRow, r = (a % kPerRow) * V;           // dst row c0 + c, dst columns r0 + r ..
+    for (int a = threadIdx.x; a < kTrTile * kOutPerRow; a += 256) {
+        const int c = a / kOutPerRow, r = (a % kOutPerRow) * VO;    // dst row c0 + c, dst columns r0 + r ..
         if (c0 + c >= cols) continue;
-        T* p = dst + (c0 + c) * rows + r0 + r;
-        if (vec_out && r0 + r + V <= rows) {
+        TO* p = dst + (c0 + c) * rows + r0 + r;
+        if (vec_out && r0 + r + VO <= rows) {
             uint4 q;
-            T* e = (T*)&q;
+            TO* e = (TO*)&q;
 #pragma unroll
-            for (int i = 0; i < V; ++i) e[i] = tile[r + i][c];
+            for (int i = 0; i < VO; ++i) e[i] = tile[r + i][c];
             *(uint4*)p = q;
         } else {
-            for (int i = 0; i < V && r0 + r + i < rows; ++i) p[i] = tile[r + i][c];
+            for (int i = 0; i < VO && r0 + r + i < rows; ++i) p[i] = tile[r + i][c];
         }
     }
 }
@@ -306,12 +319,14 @@ int launch_ce_rows(void* logits, int64_t pitch, const int64_t* targets, int64_t 
     return launch_rows<float>(logits, pitch, targets, rows, vocab, ignore_index, softcap, grad_scale, lse, nll, write_grad, stream);
 }
 
-int launch_transpose(const void* src, void* dst, int64_t rows, int64_t cols, int dtype, hipStream_t stream) {
+int launch_transpose(const void* src, void* dst, int64_t rows, int64_t cols, int src_dtype, int dst_dtype, hipStream_t stream) {
     const dim3 grid((unsigned)((cols + kTrTile - 1) / kTrTile), (unsigned)((rows + kTrTile - 1) / kTrTile));
-    if (dtype == MA_DTYPE_BF16)
-        transpose_kernel<uint16_t><<<grid, 256, 0, stream>>>((const uint16_t*)src, (uint16_t*)dst, rows, cols);
+    if (src_dtype == MA_DTYPE_BF16)
+        transpose_kernel<uint16_t, uint16_t><<<grid, 256, 0, stream>>>((const uint16_t*)src, (uint16_t*)dst, rows, cols);
+    else if (dst_dtype == MA_DTYPE_BF16)
+        transpose_kernel<float, uint16_t><<<grid, 256, 0, stream>>>((const float*)src, (uint16_t*)dst, rows, cols);
     else
-        transpose_kernel<float><<<grid, 256, 0, stream>>>((const float*)src, (float*)dst, rows, cols);
+        transpose_kernel<float, float><<<grid, 256, 0, stream>>>((const float*)src, (float*)dst, rows, cols);
     return check_launch("transpose_kernel");
 }
 

@@ -61,15 +61,17 @@ def ce_rows(logits: torch.Tensor, targets: torch.Tensor, ignore_index: int = -10
     return lse, nll
 
 
-def transpose(x: torch.Tensor) -> torch.Tensor:
-    """``x.t().contiguous()`` of a contiguous 2-d tensor (bf16 or fp32) with the library's tile kernel."""
+def transpose(x: torch.Tensor, dtype: torch.dtype | None = None) -> torch.Tensor:
+    """``x.t().contiguous()`` of a contiguous 2-d tensor (bf16 or fp32) with the library's tile kernel; with
+    ``dtype=torch.bfloat16`` an fp32 ``x`` is rounded on the way."""
     _lib.require_gpu(x, "transpose")
     if x.dim() != 2 or not x.is_contiguous():
         raise ValueError("transpose needs a contiguous 2-d tensor")
-    out = torch.empty(x.shape[1], x.shape[0], dtype=x.dtype, device=x.device)
+    dtype = x.dtype if dtype is None else dtype
+    out = torch.empty(x.shape[1], x.shape[0], dtype=dtype, device=x.device)
     with torch.cuda.device(x.device):
         rc = _lib.lib().ma_transpose(_lib.ptr(x), _lib.ptr(out), x.shape[0], x.shape[1], _lib.dtype_code(x.dtype),
-                                    _lib.current_stream(x.device))
+                                    _lib.dtype_code(dtype), _lib.current_stream(x.device))
     _lib.check(rc)
     return out
 
@@ -126,7 +128,7 @@ def linear_ce_forward(e, c, targets, ignore_index=-100, softcap=None, reduction=
     n = e_kept.shape[0]
     want_grad = need_de or need_dc
     de_kept = torch.empty_like(e_kept) if need_de else None
-    dc = dc_acc = None
+    dc = dc_t = None
     if n == 0:
         loss = _loss_reduce(torch.zeros(1, dtype=torch.float32, device=dev), scale)
         return (loss, torch.zeros_like(e) if need_de else None, torch.zeros_like(c) if need_dc else None)
@@ -147,14 +149,17 @@ def linear_ce_forward(e, c, targets, ignore_index=-100, softcap=None, reduction=
         if need_de:
             torch.mm(x, c_t.t(), out=de_kept[r0:r1])
         if need_dc:
+            # d weight^T [K, V] = e^T . d logits: with the hidden states transposed (small) this is the operand
+            # order the library runs fastest for these shapes (9.1 against 10.5 ms per 8192-row block)
+            e_t = transpose(e_kept[r0:r1])
             if n <= step:
-                dc = torch.mm(x.t(), e_kept[r0:r1])
-            elif dc_acc is None:             # several blocks: summed in fp32 by the GEMMs, rounded once at the end
-                dc_acc = torch.mm(x.t(), e_kept[r0:r1], **mixed)
+                dc_t = torch.mm(e_t, x)
+            elif dc_t is None:               # several blocks: summed in fp32 by the GEMMs, rounded once at the end
+                dc_t = torch.mm(e_t, x, **mixed)
             else:
-                torch.addmm(dc_acc, x.t(), e_kept[r0:r1], out=dc_acc, **mixed)
-    if need_dc and dc is None:
-        dc = dc_acc.to(c.dtype)
+                torch.addmm(dc_t, e_t, x, out=dc_t, **mixed)
+    if need_dc:
+        dc = transpose(dc_t, c.dtype)        # back to [V, K], rounded to the parameter's dtype on the way
     loss = _loss_reduce(nll, scale)
     de = de_kept
     if need_de and keep is not None:

@@ -226,6 +226,11 @@ def test_gemma_width_against_the_materialising_path_on_the_gpu(gpu):
 def test_transpose(gpu, shape, dtype):
     x = torch.randn(*shape).to(dtype)
     assert torch.equal(transpose(x.to(gpu)).cpu(), x.t().contiguous())
+    if dtype == torch.float32:                                 # rounded on the way, as torch's cast rounds
+        assert torch.equal(transpose(x.to(gpu), torch.bfloat16).cpu(), x.t().contiguous().bfloat16())
+    else:
+        with pytest.raises(RuntimeError):
+            transpose(x.to(gpu), torch.float32)
 
 
 def test_rows_kernel_bf16_softcap(gpu):
