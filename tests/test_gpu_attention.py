@@ -2,12 +2,13 @@
 
 Tolerances (the stated bar of the path): fp32 activations <= 1e-4 max-abs; bf16 activations
 <= 2e-2 max-abs and <= 1e-2 relative L2 against the oracle evaluated in fp32 on the same
-(bf16-rounded) inputs."""
+(bf16-rounded) inputs -- outputs and LSE flat, gradients element by element with one bf16 rounding
+of the reference value on top (``conftest.check_bf16``)."""
 import numpy as np
 import pytest
 import torch
 
-from conftest import max_abs, rel_l2
+from conftest import check_bf16, max_abs, rel_l2
 from maester_amd import build_tile_map, doc_masked_attention, packed_doc_attention, workloads
 from maester_amd.attention import attention_backward, attention_forward, backward_workspace_bytes
 from oracle import attention as A
@@ -15,7 +16,7 @@ from oracle import prologue as P
 
 pytestmark = pytest.mark.gpu
 
-BF16_MAX_ABS, BF16_REL_L2, FP32_MAX_ABS = 2e-2, 1e-2, 1e-4
+FP32_MAX_ABS = 1e-4
 
 
 def _ids(B, S, seed, kind="docs"):
@@ -40,13 +41,11 @@ def _qkv(B, S, Hq, Hkv, D, dtype, seed):
     return mk(Hq), mk(Hkv), mk(Hkv), mk(Hq)
 
 
-def _check(got, want, dtype, tag):
+def _check(got, want, dtype, tag, flat=False):
     if dtype == torch.float32:
         assert max_abs(got.cpu(), want) <= FP32_MAX_ABS, (tag, max_abs(got.cpu(), want))
     else:
-        ma, rl = max_abs(got.cpu(), want), rel_l2(got.cpu(), want)
-        scale = max(1.0, float(want.abs().max()))
-        assert ma <= BF16_MAX_ABS * scale and rl <= BF16_REL_L2, (tag, ma, rl, scale)
+        check_bf16(got, want, tag, flat=flat)
 
 
 # ------------------------------------------------------------------ fp32 path ------------------
@@ -136,7 +135,7 @@ def test_bf16_forward(gpu, case):
     tm = build_tile_map(gids, B, S, True, window, device=gpu)
     out, lse = attention_forward(q.to(gpu), k.to(gpu), v.to(gpu), tm, gids, scale, True, window)
     assert out.dtype == torch.bfloat16
-    _check(out, want, torch.bfloat16, case[0])
+    _check(out, want, torch.bfloat16, (case[0], "out"), flat=True)
     assert max_abs(lse.cpu(), wl) <= 2e-2
 
 
@@ -170,10 +169,13 @@ def test_full_path_bf16_with_norm_weights(gpu):
     hin = [g.xq.clone().requires_grad_(), g.xk.clone().requires_grad_(), g.xv.clone().requires_grad_(),
            g.q_w.clone().requires_grad_(), g.k_w.clone().requires_grad_()]
     out = packed_doc_attention(hin[0], hin[1], hin[2], hin[3], hin[4], g.cos, g.sin, g.position_ids, g.document_ids, g.scale)
-    _check(out, ref.detach(), torch.bfloat16, "out")
+    _check(out, ref.detach(), torch.bfloat16, "full path out", flat=True)
     got = torch.autograd.grad(out, hin, g.dout)
-    for name, a, b in zip(("dxq", "dxk", "dxv", "dq_w", "dk_w"), got, want):
-        _check(a, b, torch.bfloat16, name)
+    for name, a, b in zip(("dxq", "dxk", "dxv"), got[:3], want[:3]):
+        _check(a, b, torch.bfloat16, "full path " + name)
+    for name, a, b in zip(("dq_w", "dk_w"), got[3:], want[3:]):
+        # sums over B*S*H rows (values in the tens to hundreds): held relative to their size
+        assert max_abs(a.cpu(), b) <= 2e-2 * max(1.0, float(b.abs().max())) and rel_l2(a.cpu(), b) <= 1e-2, name
 
 
 @pytest.mark.parametrize("name", ["c2", "c3", "c5"])
@@ -189,7 +191,7 @@ def test_full_size_properties_and_slice(gpu, name):
     b, hk = sp.B - 1, sp.Hkv - 1
     want, wlse = A.dense_attention(q[b:b + 1, :, hk * G:(hk + 1) * G], k[b:b + 1, :, hk:hk + 1], wl.xv[b:b + 1, :, hk:hk + 1],
                                    wl.document_ids[b:b + 1], wl.scale, True, sp.window, return_lse=True)
-    _check(out[b:b + 1, :, hk * G:(hk + 1) * G], want.cpu(), torch.bfloat16, name)
+    _check(out[b:b + 1, :, hk * G:(hk + 1) * G], want.cpu(), torch.bfloat16, (name, "out slice"), flat=True)
     assert max_abs(lse[b:b + 1, hk * G:(hk + 1) * G].cpu(), wlse.cpu()) <= 2e-2
     ones = torch.ones_like(wl.xv)
     o1, _ = attention_forward(q, k, ones, tm, wl.document_ids, wl.scale, True, sp.window)
@@ -296,7 +298,7 @@ def test_full_size_backward_slices(gpu, name):
                                                    do[b:b + 1, :, hs], ids, wl.scale, True, sp.window)
         for what, got, want in (("out", out[b:b + 1, :, hs], wo), ("dq", dq[b:b + 1, :, hs], wq),
                                 ("dk", dk[b:b + 1, :, hk:hk + 1], wk), ("dv", dv[b:b + 1, :, hk:hk + 1], wv)):
-            _check(got.cpu(), want.cpu(), torch.bfloat16, (name, b, hk, what))
+            _check(got.cpu(), want.cpu(), torch.bfloat16, (name, b, hk, what), flat=(what == "out"))
         del wo, wq, wk, wv
         torch.cuda.empty_cache()
 
@@ -358,6 +360,6 @@ def test_bf16_forward_scores_that_outgrow_the_first_block(gpu, heads, D):
     gids = ids.to(gpu)
     tm = build_tile_map(gids, B, S, True, None, device=gpu)
     out, lse = attention_forward(q.to(gpu), k.to(gpu), v.to(gpu), tm, gids, scale, True, None)
-    _check(out, want, torch.bfloat16, ("outgrown", heads, D))
+    _check(out, want, torch.bfloat16, ("outgrown", heads, D), flat=True)
     assert torch.isfinite(lse).all()
     assert max_abs(lse.cpu(), wl) <= 2e-2 * max(1.0, float(wl.abs().max()) / 100)
