@@ -9,6 +9,10 @@
  *  - Every pointer is a DEVICE pointer owned by the caller (torch); the library allocates nothing,
  *    never synchronises and never throws.  Work is enqueued on `stream` (a hipStream_t passed as
  *    void*; NULL = the default stream).
+ *  - Host-side state of the library: the thread-local message behind ma_last_error(), a per-device
+ *    cache of the compute-unit count and of each kernel's occupancy (read-only after first use) and,
+ *    for ma_tile_map_build_static alone, the per-device address of its scratch array.  Device-side
+ *    state: that scratch array, and the work counters inside a caller's ma_tile_map (see there).
  *  - Every function returns MA_OK (0) or a negative MA_ERR_* code; the message of the last error of
  *    the calling thread is available from ma_last_error().  Arguments are validated before any
  *    launch, so the error paths run on a host without a GPU.
@@ -94,6 +98,19 @@ typedef struct ma_tile_map {
 size_t ma_tile_map_workspace_bytes(int B, int S);
 int ma_tile_map_build(const int64_t* document_ids, int B, int S, int causal, int64_t window,
                       const ma_tile_map* out, void* workspace, size_t workspace_bytes, void* stream);
+
+/* The same build for callers that cannot allocate (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc): no workspace argument; the scratch is a fixed array of
+ * MA_TILE_MAP_STATIC_BYTES that the library holds in device memory on every GPU it runs on until the
+ * process ends.  No counterpart in the reference.  The call allocates nothing and frees nothing;
+ * (B, S) whose ma_tile_map_workspace_bytes exceeds MA_TILE_MAP_STATIC_BYTES are rejected with
+ * MA_ERR_UNSUPPORTED (4 MiB covers B*ceil(S/128)^2 <= ~830 000 tiles, e.g. B=8 at S=32768).
+ * Every call on one GPU uses that GPU's one array (nothing in it needs to survive between calls or to
+ * be cleared by the caller): calls that overlap on one GPU -- two streams, two threads -- race; order
+ * them on one stream or with events.  Same outputs as ma_tile_map_build, bit for bit. */
+#define MA_TILE_MAP_STATIC_BYTES (4u << 20)
+int ma_tile_map_build_static(const int64_t* document_ids, int B, int S, int causal, int64_t window,
+                             const ma_tile_map* out, void* stream);
 
 /* ---- ids of packed rows ----------------------------------------------------------------------------
  * Replaces PackedSFTDataset._generate_position_ids / _generate_document_ids

@@ -22,10 +22,11 @@ MA_DTYPE_BF16 = 1
 MA_TILE = 128
 MA_DOC_BLOCK = 32
 MA_WORK_COUNTERS = 64
+MA_TILE_MAP_STATIC_BYTES = 4 << 20
 MA_BWD_DELTA, MA_BWD_DKV, MA_BWD_DQ, MA_BWD_ALL = 1, 2, 4, 7
 
 EXPORTS = (
-    "ma_version", "ma_last_error", "ma_tile_map_workspace_bytes", "ma_tile_map_build", "ma_packed_ids_build", "ma_rmsnorm_bwd_workspace_bytes", "ma_rmsnorm_fwd", "ma_rmsnorm_bwd", "ma_ce_valid_count", "ma_ce_rows", "ma_ce_loss_reduce", "ma_transpose", "ma_prologue_fwd",
+    "ma_version", "ma_last_error", "ma_tile_map_workspace_bytes", "ma_tile_map_build", "ma_tile_map_build_static", "ma_packed_ids_build", "ma_rmsnorm_bwd_workspace_bytes", "ma_rmsnorm_fwd", "ma_rmsnorm_bwd", "ma_ce_valid_count", "ma_ce_rows", "ma_ce_loss_reduce", "ma_transpose", "ma_prologue_fwd",
     "ma_prologue_bwd_workspace_bytes", "ma_prologue_bwd", "ma_attn_fwd", "ma_attn_bwd_workspace_bytes", "ma_attn_bwd_ds_workspace_bytes",
     "ma_attn_bwd", "ma_attn_bwd_stages",
 )
@@ -72,6 +73,8 @@ def lib() -> ctypes.CDLL:
     L.ma_tile_map_workspace_bytes.argtypes = [c_int, c_int]
     L.ma_tile_map_build.restype = c_int
     L.ma_tile_map_build.argtypes = [c_void_p, c_int, c_int, c_int, c_int64, TM, c_void_p, c_size_t, c_void_p]
+    L.ma_tile_map_build_static.restype = c_int
+    L.ma_tile_map_build_static.argtypes = [c_void_p, c_int, c_int, c_int, c_int64, TM, c_void_p]
     L.ma_packed_ids_build.restype = c_int
     L.ma_packed_ids_build.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]
     L.ma_rmsnorm_bwd_workspace_bytes.restype = c_size_t

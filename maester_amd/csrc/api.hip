@@ -98,19 +98,40 @@ size_t ma_tile_map_workspace_bytes(int B, int S) {
     return (((size_t)B * T * T + 15) & ~(size_t)15) + (size_t)B * T * 2 * sizeof(int64_t) + 16 + (size_t)B * T * T * sizeof(int32_t);
 }
 
-int ma_tile_map_build(const int64_t* document_ids, int B, int S, int causal, int64_t window, const ma_tile_map* out,
-                      void* workspace, size_t workspace_bytes, void* stream) {
-    const char* who = "ma_tile_map_build";
+static int check_tile_map_args(const char* who, int B, int S, int causal, int64_t window, const ma_tile_map* out) {
     if (B <= 0 || S <= 0) return fail(MA_ERR_BAD_ARG, "%s: B=%d and S=%d must be positive", who, B, S);
     if (B > 65535) return fail(MA_ERR_BAD_ARG, "%s: B=%d exceeds the grid limit 65535", who, B);
     const int64_t T = ((int64_t)S + MA_TILE - 1) / MA_TILE;
     if (T > 65535) return fail(MA_ERR_BAD_ARG, "%s: S=%d gives %lld tiles per side, limit 65535", who, S, (long long)T);
+    // tiles are numbered b*T*T + i*T + j in 32 bits (the list of tiles that need an exact count)
+    if ((int64_t)B * T * T >= ((int64_t)1 << 31))
+        return fail(MA_ERR_UNSUPPORTED, "%s: B=%d, S=%d gives %lld tiles, limit 2^31", who, B, S, (long long)((int64_t)B * T * T));
     MA_TRY(check_mask(who, causal, window));
     MA_TRY(check_map(who, out, true, true));
+    return MA_OK;
+}
+
+int ma_tile_map_build(const int64_t* document_ids, int B, int S, int causal, int64_t window, const ma_tile_map* out,
+                      void* workspace, size_t workspace_bytes, void* stream) {
+    const char* who = "ma_tile_map_build";
+    MA_TRY(check_tile_map_args(who, B, S, causal, window, out));
     if (!workspace || workspace_bytes < ma_tile_map_workspace_bytes(B, S))
         return fail(MA_ERR_BAD_ARG, "%s: workspace of %zu bytes, need %zu", who, workspace ? workspace_bytes : (size_t)0,
                     ma_tile_map_workspace_bytes(B, S));
     return launch_tile_map(document_ids, B, S, causal, window, *out, workspace, (hipStream_t)stream);
+}
+
+int ma_tile_map_build_static(const int64_t* document_ids, int B, int S, int causal, int64_t window, const ma_tile_map* out,
+                             void* stream) {
+    const char* who = "ma_tile_map_build_static";
+    MA_TRY(check_tile_map_args(who, B, S, causal, window, out));
+    const size_t need = ma_tile_map_workspace_bytes(B, S);
+    if (need > (size_t)MA_TILE_MAP_STATIC_BYTES)
+        return fail(MA_ERR_UNSUPPORTED, "%s: B=%d, S=%d needs %zu bytes of scratch, the library holds %zu; use ma_tile_map_build with a workspace",
+                    who, B, S, need, (size_t)MA_TILE_MAP_STATIC_BYTES);
+    void* ws = nullptr;
+    MA_TRY(static_tile_map_scratch(&ws));
+    return launch_tile_map(document_ids, B, S, causal, window, *out, ws, (hipStream_t)stream);
 }
 
 static int check_norm(const char* who, const void* x, const float* weight, int64_t rows, int dim, int dtype) {

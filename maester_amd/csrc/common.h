@@ -32,6 +32,8 @@ __device__ __forceinline__ bool pair_allowed(int q, int kv, int causal, int64_t 
 // Launchers (each validates nothing: the C-ABI layer in api.hip has already done so).
 int launch_tile_map(const int64_t* doc, int B, int S, int causal, int64_t window, const ma_tile_map& out,
                     void* ws, hipStream_t st);
+// device address, on the current device, of the library-owned scratch behind ma_tile_map_build_static
+int static_tile_map_scratch(void** out);
 int launch_prologue_fwd(const ma_tensor4& qi, const ma_tensor4& ki, const ma_tensor4& qo, const ma_tensor4& ko,
                         const float* qw, const float* kw, const float* cs, const float* sn, int64_t n_pos,
                         const int64_t* pos, float eps, int unit, float* q_rstd, float* k_rstd, int dtype, int B,

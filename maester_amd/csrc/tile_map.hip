@@ -9,6 +9,8 @@
 // ascending.
 #include "common.h"
 
+#include <mutex>
+
 namespace ma {
 
 // class codes in the workspace: 0 empty, 1 partial, 2 full
@@ -229,6 +231,32 @@ int launch_tile_map(const int64_t* doc, int B, int S, int causal, int64_t window
     if (!out.q_tile_order && !out.kv_tile_order) return rc;
     hipLaunchKernelGGL(schedule_kernel, dim3(2), dim3(1024), 0, st, B * T, out);
     return check_launch("schedule_kernel");
+}
+
+// ---- the build without a caller-provided workspace ----------------------------------------------------
+// Device scratch owned by the library: every GPU the library runs on holds its own copy of this array
+// until the process ends.  In host code the array's name is only a handle; its address on the current
+// device comes from hipGetSymbolAddress, once per device, and that pointer is what the kernels get.
+static __device__ __align__(256) unsigned char scratch[MA_TILE_MAP_STATIC_BYTES];
+
+static void* g_scratch_ptr[64];          // per device, written once under g_scratch_lock
+static std::mutex g_scratch_lock;
+
+int static_tile_map_scratch(void** out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(MA_ERR_LAUNCH, "ma_tile_map_build_static: hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= 64) return fail(MA_ERR_UNSUPPORTED, "ma_tile_map_build_static: device index %d (at most 64 devices)", dev);
+    std::lock_guard<std::mutex> guard(g_scratch_lock);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p)
+            return fail(MA_ERR_LAUNCH, "ma_tile_map_build_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return MA_OK;
 }
 
 }  // namespace ma

@@ -66,10 +66,12 @@ class TileMap:
 
 
 def build_tile_map(document_ids: torch.Tensor | None, batch_size: int, seq_len: int, causal: bool = True,
-                   sliding_window: int | None = None, device=None) -> TileMap:
+                   sliding_window: int | None = None, device=None, static_scratch: bool = False) -> TileMap:
     """``document_ids``: int64 [B,S] on the GPU, or ``None`` for the plain causal / sliding-window
     mask (maester/models/gemma/model.py:227-228).  ``sliding_window`` is inclusive (``q - kv <= W``,
-    model.py:206-207) and implies causality."""
+    model.py:206-207) and implies causality.  ``static_scratch``: go through ``ma_tile_map_build_static``,
+    whose scratch is a fixed array inside the library instead of a workspace allocated here (the
+    output tensors are still torch's; the C entry point itself allocates nothing)."""
     if document_ids is not None:
         _lib.require_gpu(document_ids, "build_tile_map")
         if document_ids.shape != (batch_size, seq_len):
@@ -91,9 +93,16 @@ def build_tile_map(document_ids: torch.Tensor | None, batch_size: int, seq_len: 
     if document_ids is not None:
         nblk = 2 * ((seq_len + 63) // 64)   # two 32-row blocks per 64-row step, the last step padded
         tm.block_doc_range = torch.empty(batch_size, nblk, 2, dtype=torch.int64, device=device)
+    cs = tm.c_struct()
+    if static_scratch:
+        with torch.cuda.device(device):
+            rc = L.ma_tile_map_build_static(_lib.ptr(document_ids), batch_size, seq_len, 1 if causal else 0,
+                                            -1 if sliding_window is None else int(sliding_window), byref(cs),
+                                            _lib.current_stream(device))
+        _lib.check(rc)
+        return tm
     ws_bytes = L.ma_tile_map_workspace_bytes(batch_size, seq_len)
     ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=device)
-    cs = tm.c_struct()
     with torch.cuda.device(device):
         rc = L.ma_tile_map_build(_lib.ptr(document_ids), batch_size, seq_len, 1 if causal else 0,
                                  -1 if sliding_window is None else int(sliding_window), byref(cs),

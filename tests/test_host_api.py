@@ -69,6 +69,15 @@ def test_tile_map_argument_errors():
     assert L.ma_tile_map_build(None, 1, 1024, 1, -1, ctypes.byref(m), 0x1000, 8, None) == _lib.MA_ERR_BAD_ARG
     assert "workspace" in _err()
     assert L.ma_tile_map_build(None, 1, 1024, 1, -1, ctypes.byref(m), None, 1 << 20, None) == _lib.MA_ERR_BAD_ARG
+    # tiles are numbered in 32 bits: B * T * T must stay below 2^31 (B = 1 at S = 128 * 46341 is just above)
+    assert L.ma_tile_map_build(None, 1, 128 * 46341, 1, -1, ctypes.byref(m), 0x1000, 1 << 62, None) == _lib.MA_ERR_UNSUPPORTED
+    assert "2^31" in _err()
+    # the build on the library's own scratch: the same argument checks, and sizes beyond the scratch are refused
+    assert L.ma_tile_map_build_static(None, 0, 128, 1, -1, ctypes.byref(m), None) == _lib.MA_ERR_BAD_ARG
+    assert L.ma_tile_map_build_static(None, 1, 128, 1, -1, None, None) == _lib.MA_ERR_BAD_ARG
+    assert L.ma_tile_map_workspace_bytes(16, 65536) > _lib.MA_TILE_MAP_STATIC_BYTES
+    assert L.ma_tile_map_build_static(None, 16, 65536, 1, -1, ctypes.byref(m), None) == _lib.MA_ERR_UNSUPPORTED
+    assert "scratch" in _err()
 
 
 def test_packed_ids_argument_errors():

@@ -1,0 +1,45 @@
+"""``ma_tile_map_build_static`` (the entry point that allocates nothing: its scratch is a fixed array
+inside the library) against ``ma_tile_map_build`` (caller-provided workspace), through the C ABI:
+bit-exact on every output, on two calls in a row, the second on a smaller input (the scratch keeps
+the first call's contents)."""
+from ctypes import byref
+
+import pytest
+import torch
+
+from maester_amd import _lib, build_tile_map, workloads
+
+pytestmark = pytest.mark.gpu
+
+FIELDS = ("kv_num_blocks", "kv_indices", "full_kv_num_blocks", "full_kv_indices", "q_num_blocks", "q_indices",
+          "full_q_num_blocks", "full_q_indices", "q_tile_order", "kv_tile_order", "block_doc_range", "work_counters")
+
+
+def _same(a, b):
+    for f in FIELDS:
+        x, y = getattr(a, f), getattr(b, f)
+        assert (x is None) == (y is None), f
+        if x is not None:
+            assert torch.equal(x, y), f
+
+
+def test_static_scratch_build_matches_the_workspace_build_twice_in_a_row(gpu):
+    big = workloads.make("c4").to(gpu)                      # B=2, S=16384: 164 KB of scratch
+    small = workloads.make("c2", B=1, S=1000).to(gpu)       # ragged, a fraction of the first call's scratch
+    for wl, window in ((big, None), (small, 300), (small, None)):
+        sp = wl.spec
+        want = build_tile_map(wl.document_ids, sp.B, sp.S, True, window)
+        got = build_tile_map(wl.document_ids, sp.B, sp.S, True, window, static_scratch=True)
+        torch.cuda.synchronize()
+        _same(got, want)
+    # no document ids (plain causal mask), still on the used scratch
+    _same(build_tile_map(None, 2, 700, True, 64, device=gpu, static_scratch=True), build_tile_map(None, 2, 700, True, 64, device=gpu))
+
+
+def test_static_scratch_build_rejects_what_does_not_fit(gpu):
+    L = _lib.lib()
+    B, S = 16, 65536                                        # 16 * 512^2 tiles: 21 MB of scratch
+    assert L.ma_tile_map_workspace_bytes(B, S) > _lib.MA_TILE_MAP_STATIC_BYTES
+    tm = build_tile_map(None, 1, 128, True, None, device=gpu)       # any valid struct: rejected before it is used
+    rc = L.ma_tile_map_build_static(None, B, S, 1, -1, byref(tm.c_struct()), None)
+    assert rc == _lib.MA_ERR_UNSUPPORTED and b"scratch" in L.ma_last_error()
