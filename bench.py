@@ -47,30 +47,67 @@ def time_region(fn, steps, warmup):
     return a.elapsed_time(b) / steps
 
 
-def cpu_baseline(wl, seconds_hint=20.0):
-    """The oracle (a CPU restatement: 'port') timed on the host cores on ONE (batch row, kv head)
-    slice of the same workload, forward + backward through torch autograd."""
-    from oracle import attention as OA
+def cpu_baseline(wl, budget_seconds=12.0):
+    """The reference's own CPU path on the host cores: torch's ``create_block_mask`` + eager ``flex_attention``
+    (the only CPU FlexAttention with a backward; what maester/models/gemma/model.py:384-396 calls and what
+    tests/test_packed_sft.py:148-155 run), driven by the oracle's restated mask mod, forward + backward, one
+    (batch row, kv head) slice of the workload after the other until ``budget_seconds`` of CPU work are spent
+    (a bounded sample: the whole workload is B*Hkv such slices)."""
+    from torch.nn.attention.flex_attention import create_block_mask, flex_attention
+
+    from maester_amd import workloads as W
+    from oracle import masks
     sp = wl.spec
     G = sp.Hq // sp.Hkv
-    b, hk = 0, 0
-    q = wl.xq[b:b + 1, :, hk * G:(hk + 1) * G].float()
-    k = wl.xk[b:b + 1, :, hk:hk + 1].float()
-    v = wl.xv[b:b + 1, :, hk:hk + 1].float()
-    do = wl.dout[b:b + 1, :, hk * G:(hk + 1) * G].float()
-    ids = wl.document_ids[b:b + 1]
-    t0 = time.perf_counter()
-    OA.dense_attention_fwd_bwd(q, k, v, do, ids, wl.scale, True, sp.window)
-    dt = time.perf_counter() - t0
-    from maester_amd import workloads as W
-    pairs = W.count_pairs([wl.doc_lengths[b]], sp.window)
-    flops = 12 * sp.D * G * pairs
+    slices = [(b, hk) for b in range(sp.B) for hk in range(sp.Hkv)]
+    t_mask = t_fwd = t_bwd = 0.0
+    flops = 0
+    done = 0
+    for b, hk in slices:
+        q = wl.xq[b:b + 1, :, hk * G:(hk + 1) * G].float().transpose(1, 2).requires_grad_()
+        k = wl.xk[b:b + 1, :, hk:hk + 1].float().transpose(1, 2).requires_grad_()
+        v = wl.xv[b:b + 1, :, hk:hk + 1].float().transpose(1, 2).requires_grad_()
+        do = wl.dout[b:b + 1, :, hk * G:(hk + 1) * G].float().transpose(1, 2)
+        mod = masks.make_mask_mod(wl.document_ids[b:b + 1], True, sp.window)
+        t0 = time.perf_counter()
+        bm = create_block_mask(mod, 1, None, sp.S, sp.S, device="cpu")
+        t1 = time.perf_counter()
+        o = flex_attention(q, k, v, block_mask=bm, scale=wl.scale, enable_gqa=G > 1)
+        t2 = time.perf_counter()
+        torch.autograd.grad(o, (q, k, v), do)
+        t3 = time.perf_counter()
+        t_mask, t_fwd, t_bwd = t_mask + t1 - t0, t_fwd + t2 - t1, t_bwd + t3 - t2
+        flops += 12 * sp.D * G * W.count_pairs([wl.doc_lengths[b]], sp.window)
+        done += 1
+        if t_mask + t_fwd + t_bwd >= budget_seconds:
+            break
+    dt = t_fwd + t_bwd
     return {
         "value": flops / dt / 1e12, "unit": "useful TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
-        "sample": f"oracle dense fwd+bwd (fp32, torch CPU) on 1 of {sp.B * sp.Hkv} (batch row, kv head) slices "
-                  f"of {sp.name}: S={sp.S}, G={G}, D={sp.D}; {dt:.2f} s",
-        "seconds": dt,
+        "sample": f"torch {torch.__version__} eager flex_attention fwd+bwd (fp32, CPU) with the restated mask mod on {done} of "
+                  f"{len(slices)} (batch row, kv head) slices of {sp.name} (S={sp.S}, G={G}, D={sp.D}): fwd {t_fwd:.2f} s + "
+                  f"bwd {t_bwd:.2f} s; create_block_mask for those rows {t_mask:.2f} s (not in value)",
+        "seconds": dt, "fwd_seconds": t_fwd, "bwd_seconds": t_bwd, "create_block_mask_seconds": t_mask,
+        "slices_sampled": done, "slices_in_workload": len(slices),
+        "whole_workload_seconds_extrapolated": dt * len(slices) / done,
+        "note": "value = useful FLOPs of the sampled slices / their time; the whole workload is slices_in_workload such "
+                "slices run one after the other (the factor to the whole workload is slices_in_workload / slices_sampled "
+                "in time, 1 in rate)",
     }
+
+
+def gpu_clock_mhz():
+    """The shader clock the driver reports right now (the active line of pp_dpm_sclk), or None."""
+    import glob
+    for path in sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk")):
+        try:
+            with open(path) as f:
+                for line in f:
+                    if line.rstrip().endswith("*"):
+                        return float(line.split(":")[1].strip().rstrip("*").strip().lower().replace("mhz", ""))
+        except (OSError, ValueError, IndexError):
+            continue
+    return None
 
 
 def flex_gpu_baseline(wl, q, k, steps=30, warmup=10):
@@ -212,8 +249,8 @@ def main():
     bufs = None
     if has_bwd:
         dq, dk, dv = attention_backward(q, k, wl.xv, out, wl.dout, lse, tmap, wl.document_ids, wl.scale, True, sp.window)
-        ws_bytes = backward_workspace_bytes(sp.B, sp.S, sp.Hq, sp.Hkv, sp.D, q.dtype, False if args.no_hand_over else None)
-        hand_over = ws_bytes >= _lib.lib().ma_attn_bwd_ds_workspace_bytes(sp.B, sp.S, sp.Hq, sp.Hkv, sp.D) and q.dtype == torch.bfloat16
+        ws_bytes = backward_workspace_bytes(sp.B, sp.S, sp.Hq, sp.Hkv, sp.D, q.dtype, False if args.no_hand_over else None, tmap)
+        hand_over = ws_bytes > _lib.lib().ma_attn_bwd_workspace_bytes(sp.B, sp.S, sp.Hq, sp.Hkv, sp.D) and q.dtype == torch.bfloat16
         ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
         bufs = (dq, dk, dv, ws)
 
@@ -276,6 +313,7 @@ def main():
         step()
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / K
+    clock_after = gpu_clock_mhz()
 
     vocab = 262144 if args.workload == "c1" else 262208
     loss = None if args.no_loss else loss_block(dev, sp.B * sp.S, model_dim, vocab, wl.xq.dtype, not args.no_flex_baseline)
@@ -325,7 +363,7 @@ def main():
         "pct_of_bf16_dense_peak": 100.0 * value / PEAK_BF16_DENSE_TFLOPS,
         "peak_bf16_dense_tflops": PEAK_BF16_DENSE_TFLOPS, "peak_hbm_gbps": PEAK_HBM_GBPS,
         "device": props.name, "gcn_arch": getattr(props, "gcnArchName", ""), "cus": props.multi_processor_count,
-        "clock_mhz": getattr(props, "clock_rate", 0) / 1e3,
+        "clock_mhz": clock_after, "clock_source": "pp_dpm_sclk right after the timed region (None: not readable on this box)",
         "useful_flops": fl,
         "fwd": {"ms": t_fwd, "tflops": tf(fl["fwd"], t_fwd), "pct_peak": 100 * tf(fl["fwd"], t_fwd) / PEAK_BF16_DENSE_TFLOPS},
         "bwd": None if not has_bwd else {"ms": t_bwd, "tflops": tf(fl["bwd"], t_bwd),

@@ -85,6 +85,16 @@ typedef struct ma_tile_map {
      * two of them running at once would share the counters.  May be NULL: then one workgroup is
      * launched per work item, as many as there are, and the hardware dispatcher places them. */
     int32_t* work_counters;      /* [MA_WORK_COUNTERS] */
+    /* Compact numbering of the visited tiles (not part of BlockMask): tile_slot[b,i,j] = rank of tile
+     * (q tile i, kv tile j) of batch row b among the visited (partial or full) tiles of the whole map in
+     * (b, i, j) order, -1 for a tile that is never visited; tile_count[0] = their number.  The backward
+     * indexes the dS workspace with it, which then holds visited tiles only.  Both may be NULL (no dS
+     * hand-over).  visited_tiles is the HOST copy of tile_count[0] that sizes that workspace: the
+     * caller reads it back once per map (one synchronisation per training step, the map being shared
+     * by all layers), or leaves 0: then the backward recomputes instead of handing dS over. */
+    int32_t* tile_slot;          /* [B,T,T] */
+    int32_t* tile_count;         /* [1] */
+    int64_t visited_tiles;       /* host value */
 } ma_tile_map;
 
 /* ---- block-sparse tile map --------------------------------------------------------------------
@@ -213,15 +223,15 @@ int ma_attn_fwd(const ma_tensor4* q, const ma_tensor4* k, const ma_tensor4* v, c
  * dK and dV are produced without global atomics (one workgroup owns a kv tile and walks the q-side
  * lists), so results are run-to-run deterministic.
  * workspace: at least ma_attn_bwd_workspace_bytes(...) bytes (holds delta, fp32 [B,Hq,S]).
- * With ma_attn_bwd_ds_workspace_bytes(...) bytes or more (bf16 only) the dK/dV kernel, which forms
- * dS anyway, also leaves it in the workspace (bf16, one 32 KB slot per pair of tiles and query
- * head, B*Hq*T*T slots of which only the visited ones are touched) and the dQ kernel reduces to
- * dQ = scale * dS K instead of recomputing S and dO V^T: the same dK and dV up to the summation
- * order of delta, the same dQ up to the rounding of dS to bf16 (which both variants do before the
- * product), fewer MFMAs, for a workspace that grows with T^2 (4.3 GB at B=4, S=8192, Hq=8).
- * Nothing in the workspace needs initialising. */
+ * With ma_attn_bwd_ds_workspace_bytes(...) bytes or more (bf16 only; needs map->tile_slot and
+ * map->visited_tiles) the dK/dV kernel, which forms dS anyway, also leaves it in the workspace
+ * (bf16, one 32 KB slot per VISITED pair of tiles and query head, numbered by map->tile_slot) and
+ * the dQ kernel reduces to dQ = scale * dS K instead of recomputing S and dO V^T: the same dK and dV
+ * up to the summation order of delta, the same dQ up to the rounding of dS to bf16 (which both
+ * variants do before the product), fewer MFMAs, for Hq * visited_tiles * 32 KB (0.45 GB at B=4,
+ * S=8192, Hq=8 with documents of some hundred tokens).  Nothing in the workspace needs initialising. */
 size_t ma_attn_bwd_workspace_bytes(int B, int S, int Hq, int Hkv, int D);
-size_t ma_attn_bwd_ds_workspace_bytes(int B, int S, int Hq, int Hkv, int D);
+size_t ma_attn_bwd_ds_workspace_bytes(int B, int S, int Hq, int64_t visited_tiles);
 int ma_attn_bwd(const ma_tensor4* q, const ma_tensor4* k, const ma_tensor4* v, const ma_tensor4* out,
                 const ma_tensor4* dout, const float* lse, const ma_tensor4* dq, const ma_tensor4* dk,
                 const ma_tensor4* dv, const ma_tile_map* map, const int64_t* document_ids, int causal,

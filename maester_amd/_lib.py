@@ -40,7 +40,7 @@ class MaTileMap(Structure):
     _fields_ = [(n, c_void_p) for n in (
         "kv_num_blocks", "kv_indices", "full_kv_num_blocks", "full_kv_indices",
         "q_num_blocks", "q_indices", "full_q_num_blocks", "full_q_indices", "q_tile_order", "kv_tile_order",
-        "block_doc_range", "work_counters")]
+        "block_doc_range", "work_counters", "tile_slot", "tile_count")] + [("visited_tiles", c_int64)]
 
 
 class MaesterAttnError(RuntimeError):
@@ -108,7 +108,7 @@ def lib() -> ctypes.CDLL:
     L.ma_attn_bwd_workspace_bytes.restype = c_size_t
     L.ma_attn_bwd_workspace_bytes.argtypes = [c_int] * 5
     L.ma_attn_bwd_ds_workspace_bytes.restype = c_size_t
-    L.ma_attn_bwd_ds_workspace_bytes.argtypes = [c_int] * 5
+    L.ma_attn_bwd_ds_workspace_bytes.argtypes = [c_int, c_int, c_int, c_int64]
     L.ma_attn_bwd.restype = c_int
     L.ma_attn_bwd.argtypes = [T4, T4, T4, T4, T4, c_void_p, T4, T4, T4, TM, c_void_p, c_int, c_int64, c_float,
                               c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]

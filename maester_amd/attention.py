@@ -131,19 +131,28 @@ def attention_forward(q, k, v, tile_map: TileMap, document_ids, scale, causal=Tr
     return out, lse
 
 
-# Largest workspace the backward takes for handing dS from the dK/dV kernel to the dQ kernel (bytes);
-# above it (long sequences: the slots grow with (S/128)^2) the dQ kernel recomputes S and dP instead.
+# Largest workspace the backward takes for handing dS from the dK/dV kernel to the dQ kernel (bytes), as a
+# fraction of the memory that is free when it is asked for; above it the dQ kernel recomputes S and dP instead.
 DS_WORKSPACE_LIMIT = 64 << 30
+DS_WORKSPACE_FREE_FRACTION = 0.5
 
 
-def backward_workspace_bytes(B, S, Hq, Hkv, D, dtype, hand_over=None) -> int:
-    """Workspace of ``attention_backward``: with room for dS when that fits ``DS_WORKSPACE_LIMIT`` (bf16 only);
-    ``hand_over`` True / False forces the choice."""
+def backward_workspace_bytes(B, S, Hq, Hkv, D, dtype, hand_over=None, tile_map: TileMap | None = None) -> int:
+    """Workspace of ``attention_backward``: delta alone, or delta plus one 32 KB dS slot per query head and
+    VISITED tile of ``tile_map`` (bf16 only) when that stays under ``DS_WORKSPACE_LIMIT`` and under
+    ``DS_WORKSPACE_FREE_FRACTION`` of the free device memory; ``hand_over`` True / False forces the choice."""
     L = _lib.lib()
-    small, large = L.ma_attn_bwd_workspace_bytes(B, S, Hq, Hkv, D), L.ma_attn_bwd_ds_workspace_bytes(B, S, Hq, Hkv, D)
+    small = L.ma_attn_bwd_workspace_bytes(B, S, Hq, Hkv, D)
+    if hand_over is False or dtype != torch.bfloat16 or tile_map is None or tile_map.tile_slot is None:
+        return small
+    large = L.ma_attn_bwd_ds_workspace_bytes(B, S, Hq, tile_map.visited_tiles())
+    if large == 0:
+        return small
     if hand_over is None:
-        hand_over = dtype == torch.bfloat16 and large <= DS_WORKSPACE_LIMIT
-    return large if (hand_over and dtype == torch.bfloat16) else small
+        free = torch.cuda.mem_get_info(tile_map.tile_slot.device)[0] if tile_map.tile_slot.is_cuda else 0
+        if large > DS_WORKSPACE_LIMIT or large > DS_WORKSPACE_FREE_FRACTION * free:
+            return small
+    return large
 
 
 def attention_backward(q, k, v, out, dout, lse, tile_map: TileMap, document_ids, scale, causal=True, window=None,
@@ -155,12 +164,16 @@ def attention_backward(q, k, v, out, dout, lse, tile_map: TileMap, document_ids,
     q, k, v, out, dout = (_rowmajor(t) for t in (q, k, v, out, dout))
     dev = q.device
     L = _lib.lib()
-    ws_bytes = backward_workspace_bytes(B, S, Hq, Hkv, D, q.dtype, hand_over)
     if buffers is None:
         dq = torch.empty((B, S, Hq, D), dtype=q.dtype, device=dev)
         dk = torch.empty((B, S, Hkv, D), dtype=q.dtype, device=dev)
         dv = torch.empty((B, S, Hkv, D), dtype=q.dtype, device=dev)
-        ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+        ws_bytes = backward_workspace_bytes(B, S, Hq, Hkv, D, q.dtype, hand_over, tile_map)
+        try:
+            ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+        except torch.cuda.OutOfMemoryError:      # the dS slots did not fit after all: the small workspace, recompute
+            ws_bytes = backward_workspace_bytes(B, S, Hq, Hkv, D, q.dtype, False)
+            ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
     else:
         dq, dk, dv, ws = buffers
         ws_bytes = ws.numel() * ws.element_size()

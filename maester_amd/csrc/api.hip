@@ -331,11 +331,9 @@ size_t ma_attn_bwd_workspace_bytes(int B, int S, int Hq, int Hkv, int D) {
 
 static size_t delta_bytes_aligned(int B, int S, int Hq) { return (((size_t)B * Hq * S * sizeof(float)) + 255) & ~(size_t)255; }
 
-size_t ma_attn_bwd_ds_workspace_bytes(int B, int S, int Hq, int Hkv, int D) {
-    (void)Hkv; (void)D;
-    if (B <= 0 || S <= 0 || Hq <= 0) return 0;
-    const size_t T = ((size_t)S + MA_TILE - 1) / MA_TILE;
-    return delta_bytes_aligned(B, S, Hq) + (size_t)B * Hq * T * T * MA_TILE * MA_TILE * 2;  // delta, then dS^T in bf16
+size_t ma_attn_bwd_ds_workspace_bytes(int B, int S, int Hq, int64_t visited_tiles) {
+    if (B <= 0 || S <= 0 || Hq <= 0 || visited_tiles <= 0) return 0;
+    return delta_bytes_aligned(B, S, Hq) + (size_t)Hq * (size_t)visited_tiles * MA_TILE * MA_TILE * 2;  // delta, then dS^T in bf16
 }
 
 int ma_attn_bwd(const ma_tensor4* q, const ma_tensor4* k, const ma_tensor4* v, const ma_tensor4* out,
@@ -369,9 +367,13 @@ int ma_attn_bwd_stages(const ma_tensor4* q, const ma_tensor4* k, const ma_tensor
     a.lse = (float*)lse;
     a.delta = (float*)workspace;
     a.stages = stages;
-    // a workspace large enough for dS^T selects the hand-over between the two bf16 kernels
-    if (dtype == MA_DTYPE_BF16 && workspace_bytes >= ma_attn_bwd_ds_workspace_bytes(B, S, Hq, Hkv, D))
+    // a workspace large enough for the dS^T of every visited tile selects the hand-over between the two bf16 kernels
+    const int64_t T64 = ((int64_t)S + MA_TILE - 1) / MA_TILE;
+    if (dtype == MA_DTYPE_BF16 && map->tile_slot && map->visited_tiles > 0 && map->visited_tiles <= (int64_t)B * T64 * T64 &&
+        workspace_bytes >= ma_attn_bwd_ds_workspace_bytes(B, S, Hq, map->visited_tiles)) {
         a.ds = (char*)workspace + delta_bytes_aligned(B, S, Hq);
+        a.ds_tiles = map->visited_tiles;
+    }
     return dtype == MA_DTYPE_BF16 ? launch_attn_bwd_bf16(a, (hipStream_t)stream)
                                   : launch_attn_bwd_f32(a, (hipStream_t)stream);
 }

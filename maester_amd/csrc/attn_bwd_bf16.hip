@@ -165,7 +165,8 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
         own.load(rng_row + (size_t)(min(kw_lo, a.S - 1) / MA_DOC_BLOCK) * 2);
         own.ready();
     }
-    StepTable<BM> st;
+    StepTable<BM, WRITE_DS> st;
+    if (WRITE_DS) st.numbering(a.map.tile_slot, (int64_t)b * a.T * a.T + j, a.T);     // tile (i, j) of this batch row, i walked
     {
         int lo, hi;
         visibility_limits(true, j * kTile, j * kTile + kTile - 1, BM, bounded, wlim, windowed, lo, hi);
@@ -173,7 +174,7 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
         scalar_load2(a.map.q_num_blocks + mrow, a.map.full_q_num_blocks + mrow, n_partial, n_full);
         st.init(a.map.q_indices + mrow * a.T, n_partial, a.map.full_q_indices + mrow * a.T, n_full, G, true, a.S, lo, hi,
                 blk_lo, blk_hi, rng_row, use_rng ? own.lo() : 0, use_rng ? own.hi() : 0,
-                (MA_LDS uint32_t*)(aux + 2 * BM * (4 + 4 + 8) + 16) + w * 64);
+                (MA_LDS uint32_t*)(aux + 2 * BM * (4 + 4 + 8) + 16) + w * 128);
         st.prime();
     }
 
@@ -205,7 +206,7 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
     auto issue_g = [&](int buf) { sq.issue((const __bf16*)gsrc, Gbuf(buf), w, lane, min(BM, a.S - st.r0), a.dout.stride_s); };
     const int my_runs = decltype(sq)::runs_of(w);
     bool have = st.next();
-    int q0 = st.r0, rep = st.rep;
+    int q0 = st.r0, rep = st.rep, tslot = st.tile_slot;
     bool partial = st.partial, act0 = st.act0, act1 = st.act1;
     if (have) {
         locate();
@@ -213,13 +214,12 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
         issue_g(0);
         issue_rows();
     }
-    // Where the dS^T of a step goes: slot (b, head, q tile, kv tile j) of a.ds and, inside it, the half
-    // of the q tile the step covers -- a uniform address, formed on the scalar side; the lane adds the
+    // Where the dS^T of a step goes: the slot of (head, visited tile) in a.ds and, inside it, the half of
+    // the q tile the step covers -- a uniform address, formed on the scalar side; the lane adds the
     // byte offset of its kv row and of its 8 columns, the block and the column pair are immediates.
-    auto ds_step = [&](int head, int q_first) {
-        const uint32_t slot = (((uint32_t)b * a.Hq + head) * a.T + (q_first >> 7)) * a.T + j;
-        return (char*)a.ds + (uint64_t)__builtin_amdgcn_readfirstlane(slot) * (kTile * kTile * 2) +
-               (uint32_t)__builtin_amdgcn_readfirstlane((q_first & (kTile - 1)) * 2);
+    auto ds_step = [&](int head, int q_first, int tile_slot) {
+        const uint64_t slot = (uint64_t)(uint32_t)head * (uint64_t)a.ds_tiles + (uint32_t)tile_slot;
+        return (char*)a.ds + slot * (kTile * kTile * 2) + (uint32_t)__builtin_amdgcn_readfirstlane((q_first & (kTile - 1)) * 2);
     };
     const uint32_t ds_lane = (uint32_t)((32 * w + r) * (kTile * 2) + 16 * hh);
 
@@ -240,7 +240,7 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
         const int cq0 = q0;
         const bool cpartial = partial;
         const bool skip[BM / 32] = {!act0, !act1};  // blocks in which this wave has nothing to do
-        char* ds_out = WRITE_DS ? ds_step(hk * G + rep, cq0) : nullptr;
+        char* ds_out = WRITE_DS ? ds_step(hk * G + rep, cq0, tslot) : nullptr;
         have = st.next();
         // The tile loads of the next step are spread over this step's first MFMA chains, one run
         // every few MFMAs (Q tile in the first 32-row block, dO tile in the second): issued in one
@@ -250,6 +250,7 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
         if (have) {
             q0 = st.r0;
             rep = st.rep;
+            tslot = st.tile_slot;
             partial = st.partial;
             act0 = st.act0;
             act1 = st.act1;
@@ -658,7 +659,7 @@ __device__ __forceinline__ void attn_bwd_dq_ds_bf16_item(KernArgs& a, const int 
     const int qw_lo = i * kTile + 32 * w, qw_hi = qw_lo + 31;
     const bool bounded = a.causal || a.window >= 0;
     const __bf16* kp = (const __bf16*)a.k.ptr + b * a.k.stride_b + hk * a.k.stride_h;
-    const __bf16* sp = (const __bf16*)a.ds + (((size_t)b * a.Hq + h) * a.T + i) * a.T * (kTile * kTile);   // kv tile 0 of this q tile
+    const __bf16* sp = (const __bf16*)a.ds + (size_t)h * (size_t)a.ds_tiles * (kTile * kTile);   // slot 0 of this head
     const int wlim = a.window >= 0 ? (int)min(a.window, (int64_t)0x3fffffff) : 0x7fffffff;
 
     const size_t mrow = (size_t)b * a.T + i;
@@ -672,7 +673,8 @@ __device__ __forceinline__ void attn_bwd_dq_ds_bf16_item(KernArgs& a, const int 
         own.load(rng_row + (size_t)(min(qw_lo, a.S - 1) / MA_DOC_BLOCK) * 2);
         own.ready();
     }
-    StepTable<BN> st;
+    StepTable<BN, true> st;
+    st.numbering(a.map.tile_slot, ((int64_t)b * a.T + i) * a.T, 1);     // tile (i, j) of this batch row, j walked
     {
         int lo, hi;
         visibility_limits(false, i * kTile, i * kTile + kTile - 1, BN, bounded, wlim, windowed, lo, hi);
@@ -680,7 +682,7 @@ __device__ __forceinline__ void attn_bwd_dq_ds_bf16_item(KernArgs& a, const int 
         scalar_load2(a.map.kv_num_blocks + mrow, a.map.full_kv_num_blocks + mrow, n_partial, n_full);
         st.init(a.map.kv_indices + mrow * a.T, n_partial, a.map.full_kv_indices + mrow * a.T, n_full, 1, false, a.S, lo, hi,
                 blk_lo, blk_hi, rng_row, use_rng ? own.lo() : 0, use_rng ? own.hi() : 0,
-                (MA_LDS uint32_t*)(lds0 + 2 * TL::bytes(BN) + 2 * TS::bytes(BN) + 16) + w * 64);
+                (MA_LDS uint32_t*)(lds0 + 2 * TL::bytes(BN) + 2 * TS::bytes(BN) + 16) + w * 128);
         st.prime();
     }
 
@@ -697,7 +699,7 @@ __device__ __forceinline__ void attn_bwd_dq_ds_bf16_item(KernArgs& a, const int 
     const uint32_t ksb = (uint32_t)(a.k.stride_s * 2);
     auto issue = [&](int buf) {  // K rows r0 .. r0+63 and the matching 64 rows of dS^T (row r0 of the tile list = kv row)
         sk.issue((const __bf16*)((const char*)kp + (uint64_t)(uint32_t)st.r0 * ksb), Kbuf(buf), w, lane, min(BN, a.S - st.r0), a.k.stride_s);
-        ss.issue(sp + (size_t)st.r0 * kTile, Sbuf(buf), w, lane, BN, kTile);     // slot jt, row r0 % 128: (r0 / 128) * 16384 + (r0 % 128) * 128
+        ss.issue(sp + (size_t)(uint32_t)st.tile_slot * (kTile * kTile) + (size_t)(st.r0 & (kTile - 1)) * kTile, Sbuf(buf), w, lane, BN, kTile);   // the step's 64 kv rows inside its tile's slot
     };
     bool have = st.next();
     bool act0 = st.act0, act1 = st.act1;
@@ -767,8 +769,8 @@ __device__ __forceinline__ void attn_bwd_dq_ds_pair_bf16_item(KernArgs& a, const
     const int qw_lo = i * kTile + 32 * w, qw_hi = qw_lo + 31;
     const bool bounded = a.causal || a.window >= 0;
     const __bf16* kp = (const __bf16*)a.k.ptr + b * a.k.stride_b + hk * a.k.stride_h;
-    const size_t head_slots = (size_t)a.T * a.T * (kTile * kTile);
-    const __bf16* sp0 = (const __bf16*)a.ds + (((size_t)b * a.Hq + h0) * a.T + i) * a.T * (kTile * kTile);
+    const size_t head_slots = (size_t)a.ds_tiles * (kTile * kTile);
+    const __bf16* sp0 = (const __bf16*)a.ds + (size_t)h0 * head_slots;   // slot 0 of the two heads
     const __bf16* sp1 = sp0 + head_slots;
     const int wlim = a.window >= 0 ? (int)min(a.window, (int64_t)0x3fffffff) : 0x7fffffff;
 
@@ -783,7 +785,8 @@ __device__ __forceinline__ void attn_bwd_dq_ds_pair_bf16_item(KernArgs& a, const
         own.load(rng_row + (size_t)(min(qw_lo, a.S - 1) / MA_DOC_BLOCK) * 2);
         own.ready();
     }
-    StepTable<BN> st;
+    StepTable<BN, true> st;
+    st.numbering(a.map.tile_slot, ((int64_t)b * a.T + i) * a.T, 1);     // tile (i, j) of this batch row, j walked
     {
         int lo, hi;
         visibility_limits(false, i * kTile, i * kTile + kTile - 1, BN, bounded, wlim, windowed, lo, hi);
@@ -791,7 +794,7 @@ __device__ __forceinline__ void attn_bwd_dq_ds_pair_bf16_item(KernArgs& a, const
         scalar_load2(a.map.kv_num_blocks + mrow, a.map.full_kv_num_blocks + mrow, n_partial, n_full);
         st.init(a.map.kv_indices + mrow * a.T, n_partial, a.map.full_kv_indices + mrow * a.T, n_full, 1, false, a.S, lo, hi,
                 blk_lo, blk_hi, rng_row, use_rng ? own.lo() : 0, use_rng ? own.hi() : 0,
-                (MA_LDS uint32_t*)(lds0 + 2 * kStage + 16) + w * 64);
+                (MA_LDS uint32_t*)(lds0 + 2 * kStage + 16) + w * 128);
         st.prime();
     }
 
@@ -808,8 +811,9 @@ __device__ __forceinline__ void attn_bwd_dq_ds_pair_bf16_item(KernArgs& a, const
     const uint32_t ksb = (uint32_t)(a.k.stride_s * 2);
     auto issue = [&](int buf) {
         sk.issue((const __bf16*)((const char*)kp + (uint64_t)(uint32_t)st.r0 * ksb), Kbuf(buf), w, lane, min(BN, a.S - st.r0), a.k.stride_s);
-        ss.issue(sp0 + (size_t)st.r0 * kTile, Sbuf(buf, 0), w, lane, BN, kTile);
-        ss.issue(sp1 + (size_t)st.r0 * kTile, Sbuf(buf, 1), w, lane, BN, kTile);
+        const size_t at = (size_t)(uint32_t)st.tile_slot * (kTile * kTile) + (size_t)(st.r0 & (kTile - 1)) * kTile;
+        ss.issue(sp0 + at, Sbuf(buf, 0), w, lane, BN, kTile);
+        ss.issue(sp1 + at, Sbuf(buf, 1), w, lane, BN, kTile);
     };
     const int k_runs = decltype(sk)::runs_of(w), s_runs = decltype(ss)::runs_of(w);
     bool have = st.next();
@@ -828,8 +832,9 @@ __device__ __forceinline__ void attn_bwd_dq_ds_pair_bf16_item(KernArgs& a, const
             act0 = st.act0;
             act1 = st.act1;
             ksrc = (const __bf16*)((const char*)kp + (uint64_t)(uint32_t)st.r0 * ksb);
-            s0src = sp0 + (size_t)st.r0 * kTile;
-            s1src = sp1 + (size_t)st.r0 * kTile;
+            const size_t at = (size_t)(uint32_t)st.tile_slot * (kTile * kTile) + (size_t)(st.r0 & (kTile - 1)) * kTile;
+            s0src = sp0 + at;
+            s1src = sp1 + at;
             // (smaller head dims have too few MFMAs per block to hide the runs behind: all at once)
             constexpr bool kPaced = decltype(sk)::PER <= (2 * 2 * DB) / 3 && 2 * decltype(ss)::PER <= (2 * 2 * DB) / 3;
             const bool spread = kPaced & (st.r0 + BN <= a.S) & !skip0 & !skip1;
@@ -902,7 +907,7 @@ static int bwd_dd(const AttnArgs& a, hipStream_t st) {
         rc = check_launch("attn_delta_bf16_kernel");
         if (rc) return rc;
     }
-    const size_t lds_kv = (size_t)4 * Tile<D>::bytes(kStep) + 2 * kStep * (4 + 4 + 8) + 16 + (kBwdThreads / 64) * 256;  // + work-queue box, step tables
+    const size_t lds_kv = (size_t)4 * Tile<D>::bytes(kStep) + 2 * kStep * (4 + 4 + 8) + 16 + (kBwdThreads / 64) * 512;  // + work-queue box, step tables
     if (hand_over) {
         if (a.stages & MA_BWD_DKV) {
             rc = opt_in_lds(attn_bwd_dkv_bf16_kernel<D, HAS_DOC, true>, lds_kv, "attn_bwd_dkv_bf16");
@@ -915,14 +920,14 @@ static int bwd_dd(const AttnArgs& a, hipStream_t st) {
         }
         const int G = a.Hq / a.Hkv;
         if ((a.stages & MA_BWD_DQ) && G % 2 == 0 && D >= MA_DQ_PAIR_MIN_D) {
-            const size_t lds_q = (size_t)2 * (Tile<D>::bytes(kStep) + 2 * Tile<kTile>::bytes(kStep)) + 16 + (kBwdThreads / 64) * 256;
+            const size_t lds_q = (size_t)2 * (Tile<D>::bytes(kStep) + 2 * Tile<kTile>::bytes(kStep)) + 16 + (kBwdThreads / 64) * 512;
             rc = opt_in_lds(attn_bwd_dq_ds_pair_bf16_kernel<D, HAS_DOC>, lds_q, "attn_bwd_dq_ds_pair_bf16");
             if (rc) return rc;
             hipLaunchKernelGGL((attn_bwd_dq_ds_pair_bf16_kernel<D, HAS_DOC>), dim3(work_grid(a.B * a.T, a.Hkv, G / 2), 1, 1), dim3(kBwdThreads),
                                lds_q, st, a);
             rc = check_launch("attn_bwd_dq_ds_pair_bf16_kernel");
         } else if (a.stages & MA_BWD_DQ) {
-            const size_t lds_q = (size_t)2 * Tile<D>::bytes(kStep) + 2 * Tile<kTile>::bytes(kStep) + 16 + (kBwdThreads / 64) * 256;
+            const size_t lds_q = (size_t)2 * Tile<D>::bytes(kStep) + 2 * Tile<kTile>::bytes(kStep) + 16 + (kBwdThreads / 64) * 512;
             const size_t lds_store = (size_t)(kBwdThreads / 64) * 32 * (D * 2 + 16);   // the epilogue's scratch
             const size_t lds = lds_q > lds_store ? lds_q : lds_store;
             rc = opt_in_lds(attn_bwd_dq_ds_bf16_kernel<D, HAS_DOC>, lds, "attn_bwd_dq_ds_bf16");

@@ -71,8 +71,10 @@ struct AttnArgs {
     int B, S, Hq, Hkv, D, T;
     int stages;  // MA_BWD_* mask (backward only)
     // dS^T handed from the dK/dV kernel to the dQ kernel (backward only, may be NULL): bf16
-    // [B, Hq, T, T, 128 kv, 128 q], one 32 KB slot per (q tile, kv tile) whether visited or not
+    // [Hq, ds_tiles, 128 kv, 128 q], one 32 KB slot per query head and visited (q tile, kv tile)
+    // pair, numbered by map.tile_slot
     void* ds;
+    int64_t ds_tiles;
 };
 
 // The argument block as the per-item functions of the queue-driven kernels see it: in the constant
@@ -328,7 +330,10 @@ struct StepWalk {
 // so that handing out a step is one LDS word (read a step ahead), a few bit operations and a
 // compare.  Every wave of a workgroup derives the same sequence of steps (same inputs); only the
 // two block bits are its own.  Filling takes a few vector loads and is needed once per 64 candidates.
-template <int STEP>
+// SLOTS: a second word per step, looked up in a table of tile numbers (the compact numbering of the
+// visited tiles, ma_tile_map.tile_slot) at slot_base + tile * slot_stride: the backward kernels
+// address the dS workspace with it.
+template <int STEP, bool SLOTS = false>
 struct StepTable {
     static_assert(kTile % STEP == 0 && STEP == 64, "two 32-row blocks per step");
     static constexpr int kPerTile = kTile / STEP;
@@ -339,9 +344,16 @@ struct StepTable {
     int blk_lo, blk_hi;            // ... of one of its 32-row blocks (the wave's rows)
     const int64_t* rng;            // (min, max) document id per 32-row block of the batch row, or nullptr
     int64_t own_lo, own_hi;        // id range of the wave's own rows
-    MA_LDS uint32_t* slot;         // 64 words of LDS of this wave
+    MA_LDS uint32_t* slot;         // 64 words of LDS of this wave (with SLOTS: 128, the second half for the tile numbers)
     int total, cbase, cnt, pos;
     uint32_t ahead;                // the entry after the current one (per lane copy of an LDS word)
+    const int32_t* slot_tab = nullptr;
+    int64_t slot_base = 0, slot_stride = 0;
+    uint32_t ahead_slot = 0;
+    int tile_slot = -1;            // of the current step (SLOTS)
+    __device__ __forceinline__ void numbering(const int32_t* table, int64_t base, int64_t stride) {
+        slot_tab = table; slot_base = base; slot_stride = stride;
+    }
 
     __device__ __forceinline__ void init(const int32_t* partial_list, int n_partial, const int32_t* full_list, int n_full,
                                          int repeats, bool reverse, int seq_len, int lo, int hi, int wave_lo, int wave_hi,
@@ -377,6 +389,9 @@ struct StepTable {
         const uint64_t mask = __ballot(vis);
         const int at = __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0));
         if (vis) slot[at] = word;
+        if constexpr (SLOTS) {
+            if (vis && slot_tab) slot[64 + at] = (uint32_t)slot_tab[slot_base + (int64_t)tile * slot_stride];
+        }
         cbase += 64;
         return __builtin_popcountll(mask);
     }
@@ -390,6 +405,7 @@ struct StepTable {
         while (cnt == 0 && cbase < total) cnt = fill();
         pos = 0;
         ahead = slot[0];
+        if constexpr (SLOTS) ahead_slot = slot[64];
         return cnt != 0;
     }
     __device__ __forceinline__ void prime() { refill(); }
@@ -400,8 +416,10 @@ struct StepTable {
     __device__ __forceinline__ bool next() {
         if (pos == cnt && !refill()) return false;
         const uint32_t word = __builtin_amdgcn_readfirstlane(ahead);
+        if constexpr (SLOTS) tile_slot = (int)__builtin_amdgcn_readfirstlane(ahead_slot);
         ++pos;
         ahead = slot[pos & 63];  // read now, used at the next call
+        if constexpr (SLOTS) ahead_slot = slot[64 + (pos & 63)];
         r0 = (int)(word & 0xffffffu);
         rep = (int)((word >> 24) & 31u);
         act1 = (word >> 29) & 1u;

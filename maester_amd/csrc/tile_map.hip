@@ -153,6 +153,27 @@ __global__ __launch_bounds__(64) void order_lists_kernel(const uint8_t* __restri
     if (lane == 0) *num = total;
 }
 
+// Compact numbering of the visited tiles: one wave per tile row (b, i).  The row's first slot is the
+// number of visited tiles in the rows before it (summed from the list lengths, B*T terms at most);
+// inside the row the visited tiles are numbered by ascending j.  The last row also leaves the total.
+__global__ __launch_bounds__(64) void tile_slots_kernel(const uint8_t* __restrict__ cls, int rows, int T, ma_tile_map out) {
+    const int row = blockIdx.x, lane = threadIdx.x;
+    int before = 0;
+    for (int r = lane; r < row; r += 64) before += out.kv_num_blocks[r] + out.full_kv_num_blocks[r];
+    for (int off = 32; off > 0; off >>= 1) before += __shfl_xor(before, off, 64);
+    const uint8_t* base = cls + (size_t)row * T;
+    int32_t* dst = out.tile_slot + (size_t)row * T;
+    int seen = 0;
+    for (int c0 = 0; c0 < T; c0 += 64) {
+        const int c = c0 + lane;
+        const bool set = c < T && base[c] != 0;
+        const unsigned long long m = __ballot(set);
+        if (c < T) dst[c] = set ? before + seen + __popcll(m & ((1ull << lane) - 1ull)) : -1;
+        seen += __popcll(m);
+    }
+    if (row == rows - 1 && lane == 0 && out.tile_count) *out.tile_count = before + seen;
+}
+
 // Launch schedule: the B*T tile rows ordered by descending work (number of tiles in the row's lists,
 // partial + full), ties by ascending index.  Block 0 orders the q tiles by their kv lists, block 1
 // the kv tiles by their q lists.  Rank by counting: N is small (B*T), the keys sit in LDS.
@@ -222,6 +243,11 @@ int launch_tile_map(const int64_t* doc, int B, int S, int causal, int64_t window
     hipLaunchKernelGGL(order_lists_kernel, dim3(T, B, 4), dim3(64), 0, st, cls, T, out);
     rc = check_launch("order_lists_kernel");
     if (rc) return rc;
+    if (out.tile_slot) {
+        hipLaunchKernelGGL(tile_slots_kernel, dim3(B * T), dim3(64), 0, st, cls, B * T, T, out);
+        rc = check_launch("tile_slots_kernel");
+        if (rc) return rc;
+    }
     if (doc && out.block_doc_range) {
         const int NB = 2 * ((S + 63) / 64);
         hipLaunchKernelGGL(block_ranges_kernel, dim3((B * NB + 7) / 8), dim3(256), 0, st, doc, B, S, NB, out.block_doc_range);

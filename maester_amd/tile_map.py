@@ -41,6 +41,11 @@ class TileMap:
     # work queues of the attention kernels, int32 [64], zeroed by the build (launches that share a
     # tile map must be stream-ordered); None = one workgroup per work item
     work_counters: torch.Tensor | None = None
+    # compact numbering of the visited tiles, int32 [B,T,T] (-1: never visited), and their number, int32 [1]:
+    # the backward indexes its dS workspace with it
+    tile_slot: torch.Tensor | None = None
+    tile_count: torch.Tensor | None = None
+    _visited: int | None = None
 
     NAMES = ("kv_num_blocks", "kv_indices", "full_kv_num_blocks", "full_kv_indices",
              "q_num_blocks", "q_indices", "full_q_num_blocks", "full_q_indices")
@@ -51,8 +56,15 @@ class TileMap:
     def c_struct(self) -> _lib.MaTileMap:
         ptrs = [c_void_p(getattr(self, n).data_ptr()) for n in self.NAMES]
         ptrs += [None if t is None else c_void_p(t.data_ptr()) for t in (self.q_tile_order, self.kv_tile_order, self.block_doc_range,
-                                                                           self.work_counters)]
-        return _lib.MaTileMap(*ptrs)
+                                                                           self.work_counters, self.tile_slot, self.tile_count)]
+        return _lib.MaTileMap(*ptrs, self._visited or 0)
+
+    def visited_tiles(self) -> int:
+        """Number of visited (partial or full) tiles, read back from the device on first use (one
+        synchronisation per map; the map of a training step is shared by all layers) and kept."""
+        if self._visited is None:
+            self._visited = int(self.tile_count.item()) if self.tile_count is not None else 0
+        return self._visited
 
     @property
     def seq_lengths(self):
@@ -89,7 +101,9 @@ def build_tile_map(document_ids: torch.Tensor | None, batch_size: int, seq_len: 
     tm = TileMap(nums[0], idxs[0], nums[1], idxs[1], nums[2], idxs[2], nums[3], idxs[3],
                  seq_len=seq_len, causal=bool(causal), window=sliding_window, q_tile_order=order[0],
                  kv_tile_order=order[1],
-                 work_counters=torch.empty(_lib.MA_WORK_COUNTERS, dtype=torch.int32, device=device))
+                 work_counters=torch.empty(_lib.MA_WORK_COUNTERS, dtype=torch.int32, device=device),
+                 tile_slot=torch.empty(batch_size, T, T, dtype=torch.int32, device=device),
+                 tile_count=torch.empty(1, dtype=torch.int32, device=device))
     if document_ids is not None:
         nblk = 2 * ((seq_len + 63) // 64)   # two 32-row blocks per 64-row step, the last step padded
         tm.block_doc_range = torch.empty(batch_size, nblk, 2, dtype=torch.int64, device=device)

@@ -48,12 +48,16 @@ SPECS = {
     "c4_gemma3_12b": WorkloadSpec(
         "c4_gemma3_12b", 2, 16384, 16, 8, 256, torch.bfloat16, 1e6, None, "normal", True, "bimodal_pareto", 0,
         "Gemma-3-12B layer: B=2 S=16384 Hq=16 Hkv=8 D=256 bf16, row 0 one full document, row 1 Pareto(1.2) docs"),
+    "c4s_gemma3_12b_sampled": WorkloadSpec(
+        "c4s_gemma3_12b_sampled", 2, 16384, 16, 8, 256, torch.bfloat16, 1e6, None, "normal", True, "bimodal_pareto_sampled", 0,
+        "Gemma-3-12B layer, seeded default: every row is one full document with probability 0.25 (rng.random() < 0.25), "
+        "Pareto(1.2) docs otherwise"),
     "c5_llama3_8b_shape": WorkloadSpec(
         "c5_llama3_8b_shape", 4, 8192, 32, 8, 128, torch.bfloat16, 5e5, None, "none", True, "uniform_128_4096", 0,
         "Llama-3-8B-shaped layer: B=4 S=8192 Hq=32 Hkv=8 D=128 bf16, no QK-norm, docs uniform[128,4096]"),
 }
 ALIASES = {"c1": "c1_plumbing_fp32", "c2": "c2_gemma3_4b_global", "c3": "c3_gemma3_4b_local",
-           "c4": "c4_gemma3_12b", "c5": "c5_llama3_8b_shape"}
+           "c4": "c4_gemma3_12b", "c4s": "c4s_gemma3_12b_sampled", "c5": "c5_llama3_8b_shape"}
 
 
 def spec(name: str) -> WorkloadSpec:
@@ -91,6 +95,9 @@ def document_lengths(sp: WorkloadSpec) -> list:
             # 25 % of rows hold one document that fills the row; with B=2 the fraction cannot be
             # met by sampling, so row 0 is the full-document row and the others are Pareto rows.
             rows.append([sp.S] if b == 0 else pack_row(rng, "pareto", sp.S))
+        elif sp.lengths == "bimodal_pareto_sampled":
+            # the seeded default of the same configuration: the 25 % is drawn per row
+            rows.append([sp.S] if rng.random() < 0.25 else pack_row(rng, "pareto", sp.S))
         else:
             rows.append(pack_row(rng, sp.lengths, sp.S))
     return rows

@@ -214,7 +214,7 @@ def _backward_both_ways(gpu, q, k, v, do, ids, scale, window):
     Hkv = k.shape[2]
     tm = build_tile_map(ids, B, S, True, window, device=gpu)
     out, lse = attention_forward(q, k, v, tm, ids, scale, True, window)
-    ws = torch.full((backward_workspace_bytes(B, S, Hq, Hkv, D, q.dtype, True),), 0xFF, dtype=torch.uint8, device=gpu)
+    ws = torch.full((backward_workspace_bytes(B, S, Hq, Hkv, D, q.dtype, True, tm),), 0xFF, dtype=torch.uint8, device=gpu)
     bufs = (torch.empty_like(q), torch.empty_like(k), torch.empty_like(v), ws)
     handed = attention_backward(q, k, v, out, do, lse, tm, ids, scale, True, window, buffers=bufs)
     handed = tuple(t.clone() for t in handed)
@@ -279,7 +279,7 @@ def test_full_size_ds_hand_over_reads_only_what_was_written(gpu, name):
     assert rel_l2(handed[0].float(), recomputed[0].float()) <= 2e-3
 
 
-@pytest.mark.parametrize("name", ["c2", "c3", "c4", "c5"])
+@pytest.mark.parametrize("name", ["c2", "c3", "c4", "c4s", "c5"])
 def test_full_size_backward_slices(gpu, name):
     """At the benchmark shapes: forward and backward of the whole batch through the C ABI, then two
     (row, kv head) slices of out / dq / dk / dv against the fp32 oracle evaluated on the GPU (the
@@ -300,6 +300,46 @@ def test_full_size_backward_slices(gpu, name):
                                 ("dk", dk[b:b + 1, :, hk:hk + 1], wk), ("dv", dv[b:b + 1, :, hk:hk + 1], wv)):
             _check(got.cpu(), want.cpu(), torch.bfloat16, (name, b, hk, what), flat=(what == "out"))
         del wo, wq, wk, wv
+        torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("name", ["c2", "c3", "c4"])
+def test_full_size_full_path(gpu, name):
+    """The whole path at the benchmark shape -- QK-RMSNorm with the configuration's weights, RoPE with its theta over the
+    per-document positions, attention, and the backward of all of it through ``PackedDocAttention`` -- against
+    ``oracle.attention.full_path`` in fp32 on two (row, kv head) slices (the dense score matrix of one slice is what
+    fits).  The norm-weight gradients sum over every row and head: they are checked on the loss restricted to a
+    slice, which the library sees as an upstream gradient that is zero outside the slice."""
+    wl = workloads.make(name).to(gpu)
+    sp = wl.spec
+    G = sp.Hq // sp.Hkv
+    leaves = [t.clone().requires_grad_() for t in (wl.xq, wl.xk, wl.xv, wl.q_w, wl.k_w)]
+    tm = build_tile_map(wl.document_ids, sp.B, sp.S, True, sp.window)
+    out = packed_doc_attention(*leaves, wl.cos, wl.sin, wl.position_ids, wl.document_ids, wl.scale, True, sp.window,
+                               tile_map=tm)
+    dxq, dxk, dxv = torch.autograd.grad(out, leaves[:3], wl.dout, retain_graph=True)
+    for b, hk in ((0, 0), (sp.B - 1, sp.Hkv - 1)):
+        hs = slice(hk * G, (hk + 1) * G)
+        ins = [wl.xq[b:b + 1, :, hs].float().requires_grad_(), wl.xk[b:b + 1, :, hk:hk + 1].float().requires_grad_(),
+               wl.xv[b:b + 1, :, hk:hk + 1].float().requires_grad_(), wl.q_w.clone().requires_grad_(),
+               wl.k_w.clone().requires_grad_()]
+        ref = A.full_path(ins[0], ins[1], ins[2], ins[3], ins[4], wl.cos, wl.sin, wl.position_ids[b:b + 1],
+                          wl.document_ids[b:b + 1], wl.scale, True, sp.window)
+        want = torch.autograd.grad(ref, ins, wl.dout[b:b + 1, :, hs].float())
+        _check(out[b:b + 1, :, hs], ref.detach(), torch.bfloat16, (name, "full path", b, hk, "out"), flat=True)
+        # dxq of the slice's heads depends on the slice alone; dxk / dxv of the kv head likewise (its G query heads are all in the slice)
+        for what, got, exp in (("dxq", dxq[b:b + 1, :, hs], want[0]), ("dxk", dxk[b:b + 1, :, hk:hk + 1], want[1]),
+                               ("dxv", dxv[b:b + 1, :, hk:hk + 1], want[2])):
+            _check(got, exp, torch.bfloat16, (name, "full path", b, hk, what))
+        # norm-weight gradients of the loss restricted to this slice
+        mask = torch.zeros_like(wl.dout)
+        mask[b, :, hs] = wl.dout[b, :, hs]
+        gq_w, gk_w = torch.autograd.grad(out, leaves[3:], mask, retain_graph=True)
+        for what, got, exp in (("dq_w", gq_w, want[3]), ("dk_w", gk_w, want[4])):
+            # sums over S*G rows of bf16-rounded gradients (values in the tens): held relative to their size
+            assert max_abs(got.cpu(), exp.cpu()) <= 2e-2 * max(1.0, float(exp.abs().max())) and rel_l2(got.cpu(), exp.cpu()) <= 1e-2, \
+                (name, b, hk, what, max_abs(got.cpu(), exp.cpu()), rel_l2(got.cpu(), exp.cpu()))
+        del ref, want, ins, mask
         torch.cuda.empty_cache()
 
 

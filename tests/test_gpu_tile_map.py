@@ -47,7 +47,7 @@ def test_against_torch_create_block_mask_small(gpu):
                       ("no ids", window))
 
 
-@pytest.mark.parametrize("name", ["c1", "c2", "c3", "c4", "c5"])
+@pytest.mark.parametrize("name", ["c1", "c2", "c3", "c4", "c4s", "c5"])
 def test_full_size_configs(gpu, name):
     sp = workloads.spec(name)
     rows = workloads.document_lengths(sp)
@@ -56,7 +56,8 @@ def test_full_size_configs(gpu, name):
     tm = build_tile_map(doc.to(gpu), sp.B, sp.S, True, sp.window)
     _assert_equal(tm, want, name)
     # the survey's tile census for these seeded layouts
-    census = {"c1": (35, 4), "c2": (684, 1014), "c3": (632, 752), "c4": (420, 8296), "c5": (602, 2437)}
+    census = {"c1": (35, 4), "c2": (684, 1014), "c3": (632, 752), "c4": (420, 8296), "c4s": (593, 2639),
+              "c5": (602, 2437)}      # c4: row 0 one document (forced); c4s: the seeded per-row draw of the same configuration
     assert (int(tm.kv_num_blocks.sum()), int(tm.full_kv_num_blocks.sum())) == census[name]
     assert int(tm.q_num_blocks.sum()) == census[name][0] and int(tm.full_q_num_blocks.sum()) == census[name][1]
 
@@ -107,3 +108,16 @@ def test_block_document_ranges(gpu, name, S):
     padded = np.concatenate([ids, np.repeat(ids[:, -1:], nblk * 32 - S, axis=1)], axis=1).reshape(sp.B, nblk, 32)
     assert np.array_equal(got[..., 0], padded.min(-1)) and np.array_equal(got[..., 1], padded.max(-1))
     assert build_tile_map(None, sp.B, sp.S, True, None, device=gpu).block_doc_range is None
+
+
+@pytest.mark.parametrize("name,S,window", [("c2", 8192, None), ("c3", 8192, 1024), ("c4s", 16384, None), ("c2", 1000, 64)])
+def test_compact_numbering_of_visited_tiles(gpu, name, S, window):
+    """tile_slot numbers the visited (partial or full) tiles in (b, i, j) order, -1 elsewhere; tile_count is their
+    number -- restated here from the oracle's tile classes."""
+    wl = workloads.make(name, S=S)
+    sp = wl.spec
+    tm = build_tile_map(wl.document_ids.to(gpu), sp.B, sp.S, True, window)
+    visited = (otm.tile_classes_np(wl.document_ids, sp.B, sp.S, True, window) != 0).reshape(-1)
+    want = np.where(visited, np.cumsum(visited) - 1, -1).astype(np.int32)
+    assert np.array_equal(tm.tile_slot.cpu().numpy().reshape(-1), want)
+    assert tm.visited_tiles() == int(visited.sum()) == int(tm.kv_num_blocks.sum()) + int(tm.full_kv_num_blocks.sum())

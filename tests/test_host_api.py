@@ -49,9 +49,10 @@ def test_workspace_sizes():
     assert L.ma_tile_map_workspace_bytes(0, 10) == 0
     assert L.ma_attn_bwd_workspace_bytes(4, 8192, 8, 4, 256) == 4 * 8 * 8192 * 4
     # with room for dS: delta (rounded up to 256 bytes) + one 32 KB slot per (batch row, query head, q tile, kv tile)
-    assert L.ma_attn_bwd_ds_workspace_bytes(4, 8192, 8, 4, 256) == 4 * 8 * 8192 * 4 + 4 * 8 * 64 * 64 * 32768
-    assert L.ma_attn_bwd_ds_workspace_bytes(1, 130, 2, 1, 64) == 1280 + 2 * 2 * 2 * 32768     # 1040 bytes of delta -> 1280
-    assert L.ma_attn_bwd_ds_workspace_bytes(0, 8192, 8, 4, 256) == 0
+    # delta, then one 32 KB slot per query head and VISITED tile (config 2 visits 1698 of its 16384 tiles)
+    assert L.ma_attn_bwd_ds_workspace_bytes(4, 8192, 8, 1698) == 4 * 8 * 8192 * 4 + 8 * 1698 * 32768
+    assert L.ma_attn_bwd_ds_workspace_bytes(1, 130, 2, 3) == 1280 + 2 * 3 * 32768     # 1040 bytes of delta -> 1280
+    assert L.ma_attn_bwd_ds_workspace_bytes(0, 8192, 8, 10) == 0 and L.ma_attn_bwd_ds_workspace_bytes(4, 8192, 8, 0) == 0
     assert L.ma_prologue_bwd_workspace_bytes(4, 8192, 8, 4, 256) > 0
 
 
@@ -211,8 +212,8 @@ def test_tile_map_struct_matches_the_header():
     hdr = open(os.path.join(os.path.dirname(__file__), "..", "include", "maester_attn.h")).read()
     body = hdr[hdr.index("typedef struct ma_tile_map {"):hdr.index("} ma_tile_map;")]
     body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
-    fields = re.findall(r"\b(?:int32_t|int64_t)\s*\*\s*(\w+)\s*;", body)
-    assert fields == [n for n, _ in MaTileMap._fields_] and len(fields) == 12
+    fields = re.findall(r"\b(?:int32_t|int64_t)\s*\*?\s*(\w+)\s*;", body)       # 14 device pointers, then the host count
+    assert fields == [n for n, _ in MaTileMap._fields_] and len(fields) == 15
     assert int(re.search(r"#define MA_WORK_COUNTERS (\d+)", hdr).group(1)) == _lib.MA_WORK_COUNTERS
     assert int(re.search(r"#define MA_DOC_BLOCK (\d+)", hdr).group(1)) == _lib.MA_DOC_BLOCK
 
@@ -220,15 +221,23 @@ def test_tile_map_struct_matches_the_header():
 def test_backward_workspace_choice():
     import torch
     from maester_amd import attention as A
+    from maester_amd.tile_map import TileMap
     L = _lib.lib()
-    small, large = L.ma_attn_bwd_workspace_bytes(4, 8192, 8, 4, 256), L.ma_attn_bwd_ds_workspace_bytes(4, 8192, 8, 4, 256)
-    assert A.backward_workspace_bytes(4, 8192, 8, 4, 256, torch.bfloat16) == large          # 4.3 GB: taken
-    assert A.backward_workspace_bytes(4, 8192, 8, 4, 256, torch.float32) == small           # the hand-over is a bf16 path
-    assert A.backward_workspace_bytes(4, 8192, 8, 4, 256, torch.bfloat16, hand_over=False) == small
-    assert A.backward_workspace_bytes(4, 8192, 8, 4, 256, torch.float32, hand_over=True) == small
-    # slots grow with (S / 128)^2: past the limit the dQ kernel recomputes instead
-    assert L.ma_attn_bwd_ds_workspace_bytes(8, 131072, 8, 4, 256) > A.DS_WORKSPACE_LIMIT
-    assert A.backward_workspace_bytes(8, 131072, 8, 4, 256, torch.bfloat16) == L.ma_attn_bwd_workspace_bytes(8, 131072, 8, 4, 256)
+    z = torch.zeros(1, dtype=torch.int32)
+    tm = TileMap(*([z] * 8), seq_len=8192, causal=True, window=None, tile_slot=z, tile_count=torch.tensor([1698], dtype=torch.int32))
+    assert tm.visited_tiles() == 1698
+    small, large = L.ma_attn_bwd_workspace_bytes(4, 8192, 8, 4, 256), L.ma_attn_bwd_ds_workspace_bytes(4, 8192, 8, 1698)
+    assert large - small == 8 * 1698 * 32768                                                 # 0.45 GB, a tenth of one slot per tile
+    assert A.backward_workspace_bytes(4, 8192, 8, 4, 256, torch.bfloat16, True, tm) == large
+    assert A.backward_workspace_bytes(4, 8192, 8, 4, 256, torch.float32, True, tm) == small  # the hand-over is a bf16 path
+    assert A.backward_workspace_bytes(4, 8192, 8, 4, 256, torch.bfloat16, False, tm) == small
+    assert A.backward_workspace_bytes(4, 8192, 8, 4, 256, torch.bfloat16, True, None) == small   # no map, no slots
+    # a map without visited tiles, or slots beyond the limit: the dQ kernel recomputes instead
+    tm._visited = 0
+    assert A.backward_workspace_bytes(4, 8192, 8, 4, 256, torch.bfloat16, True, tm) == small
+    tm._visited = 8 * 1024 * 1024
+    assert L.ma_attn_bwd_ds_workspace_bytes(8, 131072, 8, tm._visited) > A.DS_WORKSPACE_LIMIT
+    assert A.backward_workspace_bytes(8, 131072, 8, 4, 256, torch.bfloat16, None, tm) == L.ma_attn_bwd_workspace_bytes(8, 131072, 8, 4, 256)
 
 
 def test_text_model_mirrors_reference_parameter_names():

@@ -11,7 +11,7 @@ from maester_amd import _lib, build_tile_map, workloads
 
 pytestmark = pytest.mark.gpu
 
-FIELDS = ("kv_num_blocks", "kv_indices", "full_kv_num_blocks", "full_kv_indices", "q_num_blocks", "q_indices",
+FIELDS = ("kv_num_blocks", "kv_indices", "full_kv_num_blocks", "full_kv_indices", "q_num_blocks", "q_indices", "tile_slot", "tile_count",
           "full_q_num_blocks", "full_q_indices", "q_tile_order", "kv_tile_order", "block_doc_range", "work_counters")
 
 
