@@ -343,8 +343,8 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
                 }
             }
             // dV^T += dO^T P and dK^T += Q^T dS  (accumulators stay in AGPRs)
-            trfrag_gemm<D, 2, kBPipe, true>(lds_addr(Gs) + tbase + roff, pf, dvacc);
-            trfrag_gemm<D, 2, kBPipe, true>(lds_addr(Qs) + tbase + roff, dsf, dkacc);
+            // (one read pipeline for both products: it is filled once, and one fence serves both)
+            trfrag_gemm_two<D, 2, kBPipe>(lds_addr(Gs) + tbase + roff, pf, dvacc, lds_addr(Qs) + tbase + roff, dsf, dkacc);
         }
     }
 

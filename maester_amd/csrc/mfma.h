@@ -335,6 +335,46 @@ __device__ __forceinline__ void trfrag_gemm(uint32_t tr_addr, const bf16x8* reg_
     mfma_fence_tiles<DB, ACC_A>(acc);  // whatever comes next may read acc with the vector ALU
 }
 
+// Two products of that kind, from two LDS tiles into two sets of AGPR accumulators, as ONE read
+// pipeline: acc0[db] += L0^T x reg0[j] (MFMAs 0 .. NJ*DB-1), then acc1[db] += L1^T x reg1[j].  The
+// first fragments of the second product are requested while the last MFMAs of the first are issued,
+// so the pipeline is filled once instead of twice (a chain that starts cold waits a full LDS latency
+// for its first fragment) and one fence serves both.
+template <int D, int NJ, int P, typename Hook = NoHook>
+__device__ __forceinline__ void trfrag_gemm_two(uint32_t tr_addr0, const bf16x8* reg0_in, f32x16* acc0, uint32_t tr_addr1,
+                                                const bf16x8* reg1_in, f32x16* acc1, Hook&& hook = Hook{}) {
+    using TL = Tile<D>;
+    constexpr int DB = D / 32;
+    constexpr int H = NJ * DB;
+    constexpr int N = 2 * H;
+    bf16x8 reg0[NJ], reg1[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) { reg0[j] = reg0_in[j]; reg1[j] = reg1_in[j]; }
+    pin_frags<0, NJ>(reg0);
+    pin_frags<0, NJ>(reg1);
+    bf16x4 lo[N], hi[N];
+    auto rd = [&](auto idx) {
+        constexpr int i = decltype(idx)::value;
+        constexpr int j = (i % H) / DB, db = i % DB;
+        lo[i] = lds_read_tr16_b64<(16 * j) * TL::kPitch + db * 64>(i < H ? tr_addr0 : tr_addr1);
+        hi[i] = lds_read_tr16_b64<(16 * j + 2) * TL::kPitch + db * 64>(i < H ? tr_addr0 : tr_addr1);
+    };
+    static_for<0, (P < N ? P : N)>(rd);
+    static_for<0, N>([&](auto idx) {
+        constexpr int i = decltype(idx)::value;
+        constexpr int j = (i % H) / DB, db = i % DB;
+        constexpr int younger = (N - 1 - i) < (P - 1) ? (N - 1 - i) : (P - 1);
+        lds_wait2<2 * younger>(lo[i], hi[i]);
+        const bf16x8 f = __builtin_shufflevector(lo[i], hi[i], 0, 1, 2, 3, 4, 5, 6, 7);
+        if constexpr (i < H) mfma32_acc_a(acc0[db], f, reg0[j]);
+        else mfma32_acc_a(acc1[db], f, reg1[j]);
+        if constexpr (i + P < N) rd(std::integral_constant<int, i + P>{});
+        hook(idx);
+    });
+    mfma_fence_tiles<DB, true>(acc0);
+    pin_tiles<0, DB, true>(acc1);
+}
+
 // ---- register-blocked variants: every LDS fragment feeds two MFMAs ---------------------------------
 // For two query heads that share a kv head, the K (or V) fragment read from LDS is the same for both:
 // reading it once halves the LDS traffic per MFMA (the transposed reads of the second product are
