@@ -96,6 +96,24 @@ def cpu_baseline(wl, budget_seconds=12.0):
     }
 
 
+def mfma_probe(dev, cus):
+    """What the matrix cores sustain on this GPU under a pure MFMA load (see ma_probe_mfma): per operand pattern
+    and number of busy compute units, the shader clock held and the resulting dense bf16 rate."""
+    from maester_amd import _lib
+    L = _lib.lib()
+    out = torch.zeros(3, dtype=torch.int64, device=dev)
+    iters, res = 20000, {}
+    for label, rnd, wgs in (("ones_1cu", 0, 1), ("ones_all", 0, cus), ("random_1cu", 1, 1), ("random_all", 1, cus)):
+        for _ in range(2):      # the second run is the one kept (clocks settled)
+            _lib.check(L.ma_probe_mfma(iters, rnd, wgs, _lib.ptr(out), _lib.current_stream(dev)))
+            torch.cuda.synchronize()
+        clocks, ticks = int(out[0]), int(out[1])
+        mhz = clocks / (ticks / 100.0)
+        res[label] = {"cycles_per_mfma": clocks / (16.0 * iters), "shader_clock_mhz": mhz,
+                      "dense_bf16_tflops_all_cus": 4 * cus * 32768 / (clocks / (16.0 * iters)) * mhz * 1e6 / 1e12}
+    return res
+
+
 def gpu_clock_mhz():
     """The shader clock the driver reports right now (the active line of pp_dpm_sclk), or None."""
     import glob
@@ -202,6 +220,8 @@ def main():
     ap.add_argument("--no-hand-over", action="store_true",
                     help="backward without the dS workspace: the dQ kernel recomputes S and dP")
     ap.add_argument("--no-loss", action="store_true", help="skip the fused linear + cross-entropy block")
+    ap.add_argument("--probe", action="store_true", help="also run the MFMA probe (sustained matrix-core rate and clock under load)")
+    ap.add_argument("--no-graph", action="store_true", help="time eager launches only (no HIP graph replay of the step)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy (reference point for rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     args = ap.parse_args()
@@ -312,8 +332,48 @@ def main():
     for _ in range(K):
         step()
     torch.cuda.synchronize()
-    ms_per_step = (time.perf_counter() - t0) * 1e3 / K
+    eager_ms_per_step = ms_per_step = (time.perf_counter() - t0) * 1e3 / K
     clock_after = gpu_clock_mhz()
+
+    # The same K steps replayed from a HIP graph of one step (the library's launches are graph-safe: no
+    # allocation, no host synchronisation, no memset; the work queues reset themselves on the device).
+    # Four short kernels per step leave launch gaps that a captured step does not have.  Every replay
+    # must reproduce the eager step bit for bit; if capture is not possible the eager figure stands.
+    launch = "eager launches through the C ABI"
+    graph_error = None
+    if has_bwd and not args.no_graph:
+        try:
+            step()
+            torch.cuda.synchronize()
+            want = [t.clone() for t in (dq, dk, dv)]
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                step()
+            torch.cuda.current_stream().wait_stream(side)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                step()
+            for rep in range(3):                      # replays with eager work and synchronisations in between
+                for t in (dq, dk, dv):
+                    t.zero_()
+                graph.replay()
+                torch.cuda.synchronize()
+                if not all(torch.equal(a, b) for a, b in zip((dq, dk, dv), want)):
+                    raise RuntimeError(f"graph replay {rep} differs from the eager step")
+                step()
+                torch.cuda.synchronize()
+            for _ in range(W):
+                graph.replay()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(K):
+                graph.replay()
+            torch.cuda.synchronize()
+            ms_per_step = (time.perf_counter() - t0) * 1e3 / K
+            launch = "hipGraph replay of one captured step (ma_attn_fwd + ma_attn_bwd)"
+        except Exception as e:  # noqa: BLE001 - the eager measurement stands
+            graph_error = f"{type(e).__name__}: {str(e)[:200]}"
 
     vocab = 262144 if args.workload == "c1" else 262208
     loss = None if args.no_loss else loss_block(dev, sp.B * sp.S, model_dim, vocab, wl.xq.dtype, not args.no_flex_baseline)
@@ -359,7 +419,10 @@ def main():
         "dtype": "bf16" if sp.dtype == torch.bfloat16 else "f32", "data": "synthetic",
         "config": {"workload": sp.name, "description": sp.description, "B": sp.B, "S": sp.S, "Hq": sp.Hq,
                    "Hkv": sp.Hkv, "D": sp.D, "window": sp.window, "n_pairs": wl.n_pairs,
-                   "timed_region": "ma_attn_fwd + ma_attn_bwd (delta, dK/dV with dS hand-over, dQ) per step, inputs resident in HBM"},
+                   "timed_region": "ma_attn_fwd + ma_attn_bwd (delta, dK/dV with dS hand-over, dQ) per step, inputs resident in HBM",
+                   "launch": launch},
+        "eager_ms_per_step": eager_ms_per_step, "eager_value": total_flops / (eager_ms_per_step * 1e-3) / 1e12,
+        "graph_error": graph_error,
         "pct_of_bf16_dense_peak": 100.0 * value / PEAK_BF16_DENSE_TFLOPS,
         "peak_bf16_dense_tflops": PEAK_BF16_DENSE_TFLOPS, "peak_hbm_gbps": PEAK_HBM_GBPS,
         "device": props.name, "gcn_arch": getattr(props, "gcnArchName", ""), "cus": props.multi_processor_count,
@@ -386,6 +449,8 @@ def main():
         "linear_cross_entropy": loss,
         "roofline": roofline,
     }
+    if args.probe:
+        result["mfma_probe"] = mfma_probe(dev, props.multi_processor_count)
     if not args.no_flex_baseline and sp.dtype == torch.bfloat16:
         fx = flex_gpu_baseline(wl, q, k)
         if "fwd_bwd_ms" in fx:

@@ -97,6 +97,15 @@ typedef struct ma_tile_map {
     int64_t visited_tiles;       /* host value */
 } ma_tile_map;
 
+/* ---- device probe (measurement support; no counterpart in the reference) ---------------------------
+ * Runs `workgroups` workgroups of four waves (one per SIMD) that each issue 16 * iters
+ * v_mfma_f32_32x32x16_bf16 back to back on two accumulators, with operands of all ones or
+ * (random_data) pseudo-random values in [-1, 1].  out (device, three uint64): shader clocks and ticks
+ * of the constant 100 MHz counter that the first wave spent in the loop, and a flag that keeps the
+ * chain alive.  bench.py --probe turns them into the clock the GPU holds under that load and the
+ * MFMA rate that any kernel could sustain at most. */
+int ma_probe_mfma(int iters, int random_data, int workgroups, uint64_t* out, void* stream);
+
 /* ---- block-sparse tile map --------------------------------------------------------------------
  * Replaces create_block_mask(make_document_mask_wrapper(base, document_ids), B, None, S, S)
  * (maester/models/gemma/model.py:694-706 global, 714-730 local; torch

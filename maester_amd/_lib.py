@@ -26,7 +26,7 @@ MA_TILE_MAP_STATIC_BYTES = 4 << 20
 MA_BWD_DELTA, MA_BWD_DKV, MA_BWD_DQ, MA_BWD_ALL = 1, 2, 4, 7
 
 EXPORTS = (
-    "ma_version", "ma_last_error", "ma_tile_map_workspace_bytes", "ma_tile_map_build", "ma_tile_map_build_static", "ma_packed_ids_build", "ma_rmsnorm_bwd_workspace_bytes", "ma_rmsnorm_fwd", "ma_rmsnorm_bwd", "ma_ce_valid_count", "ma_ce_rows", "ma_ce_loss_reduce", "ma_transpose", "ma_prologue_fwd",
+    "ma_version", "ma_last_error", "ma_probe_mfma", "ma_tile_map_workspace_bytes", "ma_tile_map_build", "ma_tile_map_build_static", "ma_packed_ids_build", "ma_rmsnorm_bwd_workspace_bytes", "ma_rmsnorm_fwd", "ma_rmsnorm_bwd", "ma_ce_valid_count", "ma_ce_rows", "ma_ce_loss_reduce", "ma_transpose", "ma_prologue_fwd",
     "ma_prologue_bwd_workspace_bytes", "ma_prologue_bwd", "ma_attn_fwd", "ma_attn_bwd_workspace_bytes", "ma_attn_bwd_ds_workspace_bytes",
     "ma_attn_bwd", "ma_attn_bwd_stages",
 )
@@ -69,6 +69,8 @@ def lib() -> ctypes.CDLL:
     L.ma_version.argtypes = []
     L.ma_last_error.restype = c_char_p
     L.ma_last_error.argtypes = []
+    L.ma_probe_mfma.restype = c_int
+    L.ma_probe_mfma.argtypes = [c_int, c_int, c_int, c_void_p, c_void_p]
     L.ma_tile_map_workspace_bytes.restype = c_size_t
     L.ma_tile_map_workspace_bytes.argtypes = [c_int, c_int]
     L.ma_tile_map_build.restype = c_int

@@ -122,6 +122,7 @@ def attention_forward(q, k, v, tile_map: TileMap, document_ids, scale, causal=Tr
     lse = torch.empty((B, Hq, S), dtype=torch.float32, device=dev)
     doc = _ids(document_ids, B, S, "document_ids")
     cs = tile_map.c_struct()
+    tile_map.order_on_current_stream(dev)
     with torch.cuda.device(dev):
         rc = _lib.lib().ma_attn_fwd(
             byref(_lib.tensor4(q)), byref(_lib.tensor4(k)), byref(_lib.tensor4(v)), byref(_lib.tensor4(out)),
@@ -179,6 +180,7 @@ def attention_backward(q, k, v, out, dout, lse, tile_map: TileMap, document_ids,
         ws_bytes = ws.numel() * ws.element_size()
     doc = _ids(document_ids, B, S, "document_ids")
     cs = tile_map.c_struct()
+    tile_map.order_on_current_stream(dev)
     with torch.cuda.device(dev):
         rc = L.ma_attn_bwd_stages(
             byref(_lib.tensor4(q)), byref(_lib.tensor4(k)), byref(_lib.tensor4(v)), byref(_lib.tensor4(out)),

@@ -16,7 +16,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(HERE, "csrc", "build")
 LIB_PATH = os.path.join(HERE, "libmaester_attn.so")
 
-SOURCES = ["api.hip", "tile_map.hip", "packed_ids.hip", "rmsnorm.hip", "cross_entropy.hip", "prologue.hip", "attn_f32.hip", "attn_fwd_bf16.hip", "attn_fwd_pair_bf16.hip",
+SOURCES = ["api.hip", "probe.hip", "tile_map.hip", "packed_ids.hip", "rmsnorm.hip", "cross_entropy.hip", "prologue.hip", "attn_f32.hip", "attn_fwd_bf16.hip", "attn_fwd_pair_bf16.hip",
            "attn_bwd_bf16.hip"]
 
 # -packed-fp32-ops is switched off on purpose: fp32 arithmetic is issued as scalar-per-lane VALU

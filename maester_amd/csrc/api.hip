@@ -90,6 +90,14 @@ int ma_version(void) { return 100; }
 
 const char* ma_last_error(void) { return g_err; }
 
+int ma_probe_mfma(int iters, int random_data, int workgroups, uint64_t* out, void* stream) {
+    const char* who = "ma_probe_mfma";
+    if (iters <= 0 || iters > (1 << 20)) return fail(MA_ERR_BAD_ARG, "%s: iters=%d out of range (1 .. 2^20)", who, iters);
+    if (workgroups <= 0 || workgroups > 65535) return fail(MA_ERR_BAD_ARG, "%s: workgroups=%d out of range", who, workgroups);
+    if (!out || ((uintptr_t)out & 7) != 0) return fail(MA_ERR_BAD_ARG, "%s: out is NULL or not 8-byte aligned", who);
+    return launch_probe_mfma(iters, random_data ? 1 : 0, workgroups, (unsigned long long*)out, (hipStream_t)stream);
+}
+
 size_t ma_tile_map_workspace_bytes(int B, int S) {
     if (B <= 0 || S <= 0) return 0;
     const size_t T = ((size_t)S + MA_TILE - 1) / MA_TILE;

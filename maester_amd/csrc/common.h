@@ -94,6 +94,7 @@ __device__ __forceinline__ int fresh_tid() {
     return t;
 }
 
+int launch_probe_mfma(int iters, int random_data, int workgroups, unsigned long long* out, hipStream_t st);
 int launch_attn_fwd_f32(const AttnArgs& a, hipStream_t st);
 int launch_attn_bwd_f32(const AttnArgs& a, hipStream_t st);
 int launch_attn_fwd_bf16(const AttnArgs& a, hipStream_t st);

@@ -46,6 +46,19 @@ class TileMap:
     tile_slot: torch.Tensor | None = None
     tile_count: torch.Tensor | None = None
     _visited: int | None = None
+    _last_stream: object = None      # the torch stream of the last launch that used the work queues
+
+    def order_on_current_stream(self, device) -> None:
+        """The work queues are shared by every launch that uses this map, so two launches must never
+        overlap.  Launches on one stream are ordered anyway; when a launch comes on another stream than the
+        one before, that stream is made to wait for everything queued on the previous one."""
+        if self.work_counters is None:
+            return
+        cur = torch.cuda.current_stream(device)
+        last = self._last_stream
+        if last is not None and last != cur and not torch.cuda.is_current_stream_capturing():
+            cur.wait_stream(last)
+        self._last_stream = cur
 
     NAMES = ("kv_num_blocks", "kv_indices", "full_kv_num_blocks", "full_kv_indices",
              "q_num_blocks", "q_indices", "full_q_num_blocks", "full_q_indices")
@@ -108,6 +121,7 @@ def build_tile_map(document_ids: torch.Tensor | None, batch_size: int, seq_len: 
         nblk = 2 * ((seq_len + 63) // 64)   # two 32-row blocks per 64-row step, the last step padded
         tm.block_doc_range = torch.empty(batch_size, nblk, 2, dtype=torch.int64, device=device)
     cs = tm.c_struct()
+    tm._last_stream = torch.cuda.current_stream(device)
     if static_scratch:
         with torch.cuda.device(device):
             rc = L.ma_tile_map_build_static(_lib.ptr(document_ids), batch_size, seq_len, 1 if causal else 0,

@@ -403,3 +403,21 @@ def test_bf16_forward_scores_that_outgrow_the_first_block(gpu, heads, D):
     _check(out, want, torch.bfloat16, ("outgrown", heads, D), flat=True)
     assert torch.isfinite(lse).all()
     assert max_abs(lse.cpu(), wl) <= 2e-2 * max(1.0, float(wl.abs().max()) / 100)
+
+
+def test_launches_that_share_a_tile_map_are_ordered_across_streams(gpu):
+    """The work queues live in the tile map: a launch on another stream than the previous one is made to wait for it
+    (two overlapping launches would drain each other's queues and leave rows unwritten)."""
+    wl = workloads.make("c2", B=2, S=4096).to(gpu)
+    sp = wl.spec
+    tm = build_tile_map(wl.document_ids, sp.B, sp.S, True, None)
+    want, _ = attention_forward(wl.xq, wl.xk, wl.xv, tm, wl.document_ids, wl.scale, True, None)
+    streams = [torch.cuda.Stream() for _ in range(3)]
+    torch.cuda.synchronize()
+    outs = []
+    for rep in range(6):
+        with torch.cuda.stream(streams[rep % 3]):
+            outs.append(attention_forward(wl.xq, wl.xk, wl.xv, tm, wl.document_ids, wl.scale, True, None)[0])
+    torch.cuda.synchronize()
+    assert all(torch.equal(o, want) for o in outs)
+    assert int(tm.work_counters.abs().sum()) == 0
