@@ -335,12 +335,13 @@ def main():
     eager_ms_per_step = ms_per_step = (time.perf_counter() - t0) * 1e3 / K
     clock_after = gpu_clock_mhz()
 
-    # The same K steps replayed from a HIP graph of one step (the library's launches are graph-safe: no
-    # allocation, no host synchronisation, no memset; the work queues reset themselves on the device).
-    # Four short kernels per step leave launch gaps that a captured step does not have.  Every replay
-    # must reproduce the eager step bit for bit; if capture is not possible the eager figure stands.
+    # Informational: the same K steps replayed from a HIP graph of one step (the library's launches are
+    # graph-safe: no allocation, no host synchronisation, no memset; the work queues reset themselves on
+    # the device).  Every replay must reproduce the eager step bit for bit.  The headline stays the eager
+    # figure: at ~1 ms per step the four launches are queued far ahead of the GPU either way.
     launch = "eager launches through the C ABI"
     graph_error = None
+    graph_ms_per_step = None
     if has_bwd and not args.no_graph:
         try:
             step()
@@ -370,8 +371,7 @@ def main():
             for _ in range(K):
                 graph.replay()
             torch.cuda.synchronize()
-            ms_per_step = (time.perf_counter() - t0) * 1e3 / K
-            launch = "hipGraph replay of one captured step (ma_attn_fwd + ma_attn_bwd)"
+            graph_ms_per_step = (time.perf_counter() - t0) * 1e3 / K
         except Exception as e:  # noqa: BLE001 - the eager measurement stands
             graph_error = f"{type(e).__name__}: {str(e)[:200]}"
 
@@ -421,8 +421,8 @@ def main():
                    "Hkv": sp.Hkv, "D": sp.D, "window": sp.window, "n_pairs": wl.n_pairs,
                    "timed_region": "ma_attn_fwd + ma_attn_bwd (delta, dK/dV with dS hand-over, dQ) per step, inputs resident in HBM",
                    "launch": launch},
-        "eager_ms_per_step": eager_ms_per_step, "eager_value": total_flops / (eager_ms_per_step * 1e-3) / 1e12,
-        "graph_error": graph_error,
+        "hip_graph_replay": {"ms_per_step": graph_ms_per_step, "error": graph_error,
+                             "value": None if graph_ms_per_step is None else total_flops / (graph_ms_per_step * 1e-3) / 1e12},
         "pct_of_bf16_dense_peak": 100.0 * value / PEAK_BF16_DENSE_TFLOPS,
         "peak_bf16_dense_tflops": PEAK_BF16_DENSE_TFLOPS, "peak_hbm_gbps": PEAK_HBM_GBPS,
         "device": props.name, "gcn_arch": getattr(props, "gcnArchName", ""), "cus": props.multi_processor_count,
