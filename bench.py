@@ -220,6 +220,9 @@ def main():
     ap.add_argument("--no-hand-over", action="store_true",
                     help="backward without the dS workspace: the dQ kernel recomputes S and dP")
     ap.add_argument("--no-loss", action="store_true", help="skip the fused linear + cross-entropy block")
+    ap.add_argument("--settle-seconds", type=float, default=2.0,
+                    help="run untimed steps for this long before anything is timed, so that the clocks are at their steady state "
+                         "whatever --warmup is (a GPU coming out of idle runs its first ~50 steps 5-8 %% slower)")
     ap.add_argument("--probe", action="store_true", help="also run the MFMA probe (sustained matrix-core rate and clock under load)")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches only (no HIP graph replay of the step)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -286,7 +289,14 @@ def main():
         if has_bwd:
             bwd()
 
-    # per-kernel durations first (HIP events on the launch stream); the headline region below then
+    # steady state first: untimed steps for --settle-seconds
+    t_settle = time.perf_counter()
+    while time.perf_counter() - t_settle < args.settle_seconds:
+        for _ in range(20):
+            step()
+        torch.cuda.synchronize()
+
+    # per-kernel durations next (HIP events on the launch stream); the headline region below then
     # starts on a device that is already at its working clocks
     t_fwd = time_region(fwd, K, W)
     t_delta = t_dkv = t_dq = t_bwd = None
@@ -325,6 +335,12 @@ def main():
     del nx, nres, ndy
 
     # ---- the headline region: W untimed steps, then exactly K timed steps ----------------------------
+    # (the passes above left the GPU in another power state: back to the steady state of the step first)
+    t_settle = time.perf_counter()
+    while time.perf_counter() - t_settle < args.settle_seconds / 2:
+        for _ in range(20):
+            step()
+        torch.cuda.synchronize()
     for _ in range(W):
         step()
     torch.cuda.synchronize()
@@ -425,6 +441,7 @@ def main():
                              "value": None if graph_ms_per_step is None else total_flops / (graph_ms_per_step * 1e-3) / 1e12},
         "pct_of_bf16_dense_peak": 100.0 * value / PEAK_BF16_DENSE_TFLOPS,
         "peak_bf16_dense_tflops": PEAK_BF16_DENSE_TFLOPS, "peak_hbm_gbps": PEAK_HBM_GBPS,
+        "settle_seconds": args.settle_seconds,
         "device": props.name, "gcn_arch": getattr(props, "gcnArchName", ""), "cus": props.multi_processor_count,
         "clock_mhz": clock_after, "clock_source": "pp_dpm_sclk right after the timed region (None: not readable on this box)",
         "useful_flops": fl,
