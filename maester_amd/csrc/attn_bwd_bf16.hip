@@ -25,9 +25,32 @@
 
 namespace ma {
 
+#ifdef MA_TICKS
+// debug build only: cycles a wave spends between two marked points of the dK/dV kernel
+__device__ unsigned long long ma_dbg_ticks[4];
+struct Ticks {
+    unsigned long long begin = 0, acc = 0;
+    unsigned n = 0;
+    bool armed = false;
+    template <int ID>
+    __device__ __forceinline__ void at() {
+        if constexpr (ID == MA_T_END) {
+            if (armed) { acc += __builtin_readcyclecounter() - begin; ++n; armed = false; }
+        }
+        if constexpr (ID == MA_T_BEGIN) { begin = __builtin_readcyclecounter(); armed = true; }
+    }
+};
+#define MA_TICK(id) ticks.template at<id>()
+#else
+#define MA_TICK(id)
+#endif
+
 constexpr int kBwdThreads = 256;
 constexpr int kStep = 64;   // rows staged per step
-constexpr int kBPipe = 4;   // LDS fragment reads kept in flight ahead of the MFMAs
+#ifndef MA_BPIPE
+#define MA_BPIPE 4
+#endif
+constexpr int kBPipe = MA_BPIPE;   // LDS fragment reads kept in flight ahead of the MFMAs
 
 // O tile epilogue shared by the kernels: a wave holds a 32-row x D fp32 tile transposed in registers
 // (lane (r, hh) owns row r and, per 32-column block, columns 8g + 4hh + e); it is scaled, cast to
@@ -87,10 +110,131 @@ __global__ __launch_bounds__(256) void attn_delta_bf16_kernel(AttnArgs a) {
 // ------------------------------------------------------------------------------------------------
 // dK / dV
 // ------------------------------------------------------------------------------------------------
+// The q-side steps of one dK/dV work item, resolved ahead of the loop that runs them.  A wave that has
+// its SIMD to itself pays four cycles for every instruction it issues between two MFMA chains, so
+// whatever a step needs is worked out 64 steps at a time, one candidate step per lane, and kept as a
+// record of ready-made addresses in the wave's own slice of LDS; taking a step is then three
+// broadcast LDS reads and a dozen v_readfirstlane.
+//   word 0       first q row | query head within the group << 24 | act1 << 29 | act0 << 30 | partial << 31
+//                (act0 / act1: this wave has something to do in the first / second 32-row block)
+//   words 2,3    address of the step's first Q row        words 4,5    of its first dO row
+//   words 6,7    of its first lse entry                   words 8,9    of its first delta entry
+//   words 10,11  of its dS^T slab in the workspace (WRITE_DS)
+// Every wave of a workgroup derives the same sequence of steps (same inputs); only the two block
+// bits are its own.  Nothing a refill needs is kept between refills except the position in the walk:
+// it is derived again from the argument block, so that the step loop holds no registers for it.
+// Which chain of a step carries which of the next step's tile loads, in eighths of a wave's runs:
+// kDkvPlan[block][chain (0: S / dP, 1: dV / dK)] = {tile (0: Q, 1: dO), first eighth, eighths}.
+#ifndef MA_DKV_PLACE
+#define MA_DKV_PLACE 0
+#endif
+#if MA_DKV_PLACE == 0
+constexpr int kDkvPlan[2][2][3] = {{{0, 0, 8}, {0, 0, 0}}, {{1, 0, 8}, {0, 0, 0}}};
+#elif MA_DKV_PLACE == 1
+constexpr int kDkvPlan[2][2][3] = {{{0, 0, 8}, {1, 0, 8}}, {{0, 0, 0}, {0, 0, 0}}};
+#elif MA_DKV_PLACE == 2
+constexpr int kDkvPlan[2][2][3] = {{{0, 0, 8}, {1, 0, 4}}, {{1, 4, 4}, {0, 0, 0}}};
+#elif MA_DKV_PLACE == 3
+constexpr int kDkvPlan[2][2][3] = {{{0, 0, 4}, {0, 4, 4}}, {{1, 0, 4}, {1, 4, 4}}};
+#endif
+constexpr int kDkvRecWords = 12;
+constexpr int kDkvRecBytes = 64 * kDkvRecWords * 4;  // LDS per wave
+template <bool HAS_DOC, bool WRITE_DS>
+struct DkvSteps {
+    MA_LDS uint32_t* tab;
+    int cbase, cnt, pos;
+    __device__ __forceinline__ void start(MA_LDS uint32_t* table) { tab = table; cbase = 0; cnt = 0; pos = -1; }
+
+    // the next candidates that hold a step at all; false when the walk is over
+    __device__ __forceinline__ bool refill(const int j, const int hk, const int b, const int w) {
+        KernArgs& a = fresh_args();
+        const int lane = __lane_id();
+        const int G = a.Hq / a.Hkv;
+        const size_t mrow = (size_t)b * a.T + j;
+        int np, nf;
+        scalar_load2(a.map.q_num_blocks + mrow, a.map.full_q_num_blocks + mrow, np, nf);
+        const int n = np + nf, per_pass = n * (kTile / kStep), total = per_pass * G;
+        const bool bounded = a.causal || a.window >= 0, windowed = a.window >= 0;
+        const int wlim = windowed ? (int)min(a.window, (int64_t)0x3fffffff) : 0x7fffffff;
+        const int kw_lo = j * kTile + 32 * w, kw_hi = kw_lo + 31;
+        int vis_lo, vis_hi, blk_lo, blk_hi;
+        visibility_limits(true, j * kTile, j * kTile + kTile - 1, kStep, bounded, wlim, windowed, vis_lo, vis_hi);
+        visibility_limits(true, kw_lo, kw_hi, 32, bounded, wlim, windowed, blk_lo, blk_hi);
+        const bool use_rng = HAS_DOC && a.map.block_doc_range != nullptr;
+        const int64_t* rng = use_rng ? a.map.block_doc_range + (size_t)b * (2 * ((a.S + 63) / 64)) * 2 : nullptr;
+        int64_t own_lo = 0, own_hi = 0;
+        if (use_rng) {
+            DocRange own;
+            own.load(rng + (size_t)(min(kw_lo, a.S - 1) / MA_DOC_BLOCK) * 2);
+            own.ready();
+            own_lo = own.lo();
+            own_hi = own.hi();
+        }
+        const int32_t* pl = a.map.q_indices + mrow * a.T;
+        const int32_t* fl = a.map.full_q_indices + mrow * a.T;
+        cnt = 0;
+        while (cnt == 0 && cbase < total) {
+            const int c = cbase + lane;
+            const bool valid = c < total;
+            const int cc = valid ? c : 0;
+            const int rep = cc / per_pass, wi = cc - rep * per_pass;
+            const int it = wi / (kTile / kStep), half = wi - it * (kTile / kStep);
+            const int idx = n - 1 - it;  // from the last q tile down: the workgroups of a document start on the same tiles
+            const bool partial = idx < np;
+            int tile = 0;
+            if (valid) tile = partial ? pl[idx] : fl[idx - np];
+            const int r0 = tile * kTile + half * kStep;
+            const bool vis = valid & (r0 < a.S) & (!partial | ((r0 >= vis_lo) & (r0 <= vis_hi)));
+            bool act0 = (r0 < a.S) & (!partial | ((r0 >= blk_lo) & (r0 <= blk_hi)));
+            bool act1 = (r0 + 32 < a.S) & (!partial | ((r0 + 32 >= blk_lo) & (r0 + 32 <= blk_hi)));
+            if (use_rng && partial && vis) {  // no row of the block shares a document with the wave's own rows
+                const int64_t* e = rng + (size_t)(r0 / 32) * 2;
+                act0 &= (e[0] <= own_hi) & (e[1] >= own_lo);
+                act1 &= (e[2] <= own_hi) & (e[3] >= own_lo);
+            }
+            const uint64_t mask = __ballot(vis);
+            const int at = __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0));
+            if (vis) {
+                const int h = hk * G + rep;
+                const uint64_t qa = (uint64_t)((const __bf16*)a.q.ptr + b * a.q.stride_b + h * a.q.stride_h + (int64_t)r0 * a.q.stride_s);
+                const uint64_t ga = (uint64_t)((const __bf16*)a.dout.ptr + b * a.dout.stride_b + h * a.dout.stride_h + (int64_t)r0 * a.dout.stride_s);
+                const size_t row = ((size_t)b * a.Hq + h) * a.S + r0;
+                const uint64_t la = (uint64_t)(a.lse + row), ea = (uint64_t)(a.delta + row);
+                uint64_t da = 0;
+                if (WRITE_DS) {
+                    const uint32_t tslot = (uint32_t)a.map.tile_slot[((int64_t)b * a.T + tile) * a.T + j];
+                    da = (uint64_t)((char*)a.ds + ((uint64_t)(uint32_t)h * (uint64_t)a.ds_tiles + tslot) * (kTile * kTile * 2) + (r0 & (kTile - 1)) * 2);
+                }
+                MA_LDS uint32_t* rec = tab + at * kDkvRecWords;
+                *(MA_LDS u32x4*)rec = u32x4{(uint32_t)r0 | ((uint32_t)rep << 24) | ((uint32_t)act1 << 29) | ((uint32_t)act0 << 30) | ((uint32_t)partial << 31),
+                                            0u, (uint32_t)qa, (uint32_t)(qa >> 32)};
+                *(MA_LDS u32x4*)(rec + 4) = u32x4{(uint32_t)ga, (uint32_t)(ga >> 32), (uint32_t)la, (uint32_t)(la >> 32)};
+                *(MA_LDS u32x4*)(rec + 8) = u32x4{(uint32_t)ea, (uint32_t)(ea >> 32), (uint32_t)da, (uint32_t)(da >> 32)};
+            }
+            cbase += 64;
+            cnt = __builtin_popcountll(mask);
+        }
+        pos = 0;
+        return cnt != 0;
+    }
+    // moves on to the next step: false when the walk is over
+    __device__ __forceinline__ bool advance(const int j, const int hk, const int b, const int w) {
+        if (++pos < cnt) return true;
+        return refill(j, hk, b, w);
+    }
+};
+__device__ __forceinline__ uint64_t uniform64(uint32_t lo, uint32_t hi) {
+    return (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane(lo) | ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane(hi) << 32);
+}
+
 // WRITE_DS: every 32 x 32 block of every step the workgroup walks also leaves its dS^T in a.ds (zeros
 // for a block the wave skips), for the dQ kernel that only multiplies it with K.
 template <int D, bool HAS_DOC, bool WRITE_DS>
-__device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg_id) {
+__device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg_id
+#ifdef MA_TICKS
+    , Ticks& ticks
+#endif
+) {
     using TL = Tile<D>;
     constexpr int KK = D / 16;
     constexpr int DB = D / 32;
@@ -112,17 +256,17 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
     int j, hk, b;
     if (!map_work(wg_id, a.B * a.T, a.T, a.Hkv, 1, a.map.kv_tile_order, j, hk, b)) return;
     const int rbase = TL::row_base(lane), tbase = TL::tr_base(lane);
-    const int G = a.Hq / a.Hkv;
-    const int kw_lo = j * kTile + 32 * w, kw_hi = kw_lo + 31;
+    const int kw_lo = j * kTile + 32 * w;
     const int kv = kw_lo + r;
     const bool kvalid = kv < a.S;
     const bool bounded = a.causal || a.window >= 0;
     const float sl2 = a.scale * kLog2e;
+    const int S = a.S;
 
     const __bf16* kp = (const __bf16*)a.k.ptr + b * a.k.stride_b + hk * a.k.stride_h;
     const __bf16* vp = (const __bf16*)a.v.ptr + b * a.v.stride_b + hk * a.v.stride_h;
-    const int64_t* drow = HAS_DOC ? a.doc + (size_t)b * a.S : nullptr;
-    const int kvc = min(kv, a.S - 1);
+    const int64_t* drow = HAS_DOC ? a.doc + (size_t)b * S : nullptr;
+    const int kvc = min(kv, S - 1);
     const int64_t dock = HAS_DOC ? drow[kvc] : 0;
     const int wlim = a.window >= 0 ? (int)min(a.window, (int64_t)0x3fffffff) : 0x7fffffff;
 
@@ -132,7 +276,7 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
         DirectStager<D, kTile, NW> sk, sv;
         sk.init(w, lane);
         sv.init(w, lane);
-        const int rows_valid = min(kTile, a.S - j * kTile);
+        const int rows_valid = min(kTile, S - j * kTile);
         sk.issue(kp + (int64_t)j * kTile * a.k.stride_s, Qbuf(0), w, lane, rows_valid, a.k.stride_s);
         sv.issue(vp + (int64_t)j * kTile * a.v.stride_s, Qbuf(1), w, lane, rows_valid, a.v.stride_s);
         wait_vmem();
@@ -151,149 +295,171 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
 #pragma unroll
         for (int v = 0; v < 16; ++v) dkacc[db][v] = dvacc[db][v] = 0.f;
 
-    const size_t mrow = (size_t)b * a.T + j;
-    // q steps of the kv tile, for each of the G query heads in turn, from the last q tile down (see
-    // ListWalk); limits inside which a 32-row q block of a partial tile can be visible to this wave
-    const bool windowed = a.window >= 0;
-    int blk_lo, blk_hi;
-    visibility_limits(true, kw_lo, kw_hi, 32, bounded, wlim, windowed, blk_lo, blk_hi);
-    // document-id range of the wave's own kv rows (the step table tests the q blocks against it)
-    const bool use_rng = HAS_DOC && a.map.block_doc_range != nullptr;
-    const int64_t* rng_row = use_rng ? a.map.block_doc_range + (size_t)b * (2 * ((a.S + 63) / 64)) * 2 : nullptr;
-    DocRange own;
-    if (use_rng) {
-        own.load(rng_row + (size_t)(min(kw_lo, a.S - 1) / MA_DOC_BLOCK) * 2);
-        own.ready();
-    }
-    StepTable<BM, WRITE_DS> st;
-    if (WRITE_DS) st.numbering(a.map.tile_slot, (int64_t)b * a.T * a.T + j, a.T);     // tile (i, j) of this batch row, i walked
-    {
-        int lo, hi;
-        visibility_limits(true, j * kTile, j * kTile + kTile - 1, BM, bounded, wlim, windowed, lo, hi);
-        int n_partial, n_full;
-        scalar_load2(a.map.q_num_blocks + mrow, a.map.full_q_num_blocks + mrow, n_partial, n_full);
-        st.init(a.map.q_indices + mrow * a.T, n_partial, a.map.full_q_indices + mrow * a.T, n_full, G, true, a.S, lo, hi,
-                blk_lo, blk_hi, rng_row, use_rng ? own.lo() : 0, use_rng ? own.hi() : 0,
-                (MA_LDS uint32_t*)(aux + 2 * BM * (4 + 4 + 8) + 16) + w * 128);
-        st.prime();
-    }
+    DkvSteps<HAS_DOC, WRITE_DS> st;
+    st.start((MA_LDS uint32_t*)(aux + 2 * BM * (4 + 4 + 8) + 16) + w * (kDkvRecBytes / 4));
 
-    DirectStager<D, BM, NW> sq;  // the Q and dO tiles have the same shape: one set of slots
+    // The Q and dO tiles have the same shape: one set of slots.  Every wave moves the same number of runs
+    // of a tile from inside its MFMA chains (kPaced, one every four MFMAs); the run that is left over
+    // (a tile is 4 * kPaced + 1 runs) is moved by wave 0 (Q) or wave 1 (dO) when the step begins.
+    using SQ = DirectStager<D, BM, NW>;
+    constexpr int kPaced = (SQ::NL - 1) / NW;
+    static_assert(SQ::NL == NW * kPaced + 1 && (2 * KK) % kPaced == 0, "tile runs per wave");
+    constexpr int kEvery = (2 * KK) / kPaced;
+    SQ sq;
     sq.init(w, lane);
-    const uint32_t qsb = (uint32_t)(a.q.stride_s * 2), gsb = (uint32_t)(a.dout.stride_s * 2);  // row strides in bytes
-    const char* qhead = (const char*)((const __bf16*)a.q.ptr + b * a.q.stride_b);
-    const char* ghead = (const char*)((const __bf16*)a.dout.ptr + b * a.dout.stride_b);
-    float lse_next = 0.f, dl_next = 0.f;
-    int64_t qd_next = 0;
-    // global sources of the step the iterator stands on
-    const char *qsrc = nullptr, *gsrc = nullptr;
-    auto locate = [&]() {
-        const int h = hk * G + st.rep;
-        qsrc = qhead + (uint64_t)(uint32_t)h * (uint32_t)(a.q.stride_h * 2) + (uint64_t)(uint32_t)st.r0 * qsb;
-        gsrc = ghead + (uint64_t)(uint32_t)h * (uint32_t)(a.dout.stride_h * 2) + (uint64_t)(uint32_t)st.r0 * gsb;
-    };
-    auto issue_rows = [&]() {  // per-row lse / delta / document id of that step
-        if (tid < BM) {
-            const int h = hk * G + st.rep;
-            const int qq = min(st.r0 + tid, a.S - 1);
-            const size_t row = ((size_t)b * a.Hq + h) * a.S + qq;
-            lse_next = a.lse[row];  // converted to log2 units when it is written to LDS
-            dl_next = a.delta[row];
-            if (HAS_DOC) qd_next = drow[qq];
-        }
-    };
-    auto issue_q = [&](int buf) { sq.issue((const __bf16*)qsrc, Qbuf(buf), w, lane, min(BM, a.S - st.r0), a.q.stride_s); };
-    auto issue_g = [&](int buf) { sq.issue((const __bf16*)gsrc, Gbuf(buf), w, lane, min(BM, a.S - st.r0), a.dout.stride_s); };
-    const int my_runs = decltype(sq)::runs_of(w);
-    bool have = st.next();
-    int q0 = st.r0, rep = st.rep, tslot = st.tile_slot;
-    bool partial = st.partial, act0 = st.act0, act1 = st.act1;
-    if (have) {
-        locate();
-        issue_q(0);
-        issue_g(0);
-        issue_rows();
+    uint32_t rc_last;  // the left-over run, whichever wave moves it
+    {
+        int row, chunk;
+        SQ::slot(SQ::NL - 1, lane, row, chunk);
+        rc_last = (uint32_t)(row << 16 | chunk * 16);
     }
-    // Where the dS^T of a step goes: the slot of (head, visited tile) in a.ds and, inside it, the half of
-    // the q tile the step covers -- a uniform address, formed on the scalar side; the lane adds the
-    // byte offset of its kv row and of its 8 columns, the block and the column pair are immediates.
-    auto ds_step = [&](int head, int q_first, int tile_slot) {
-        const uint64_t slot = (uint64_t)(uint32_t)head * (uint64_t)a.ds_tiles + (uint32_t)tile_slot;
-        return (char*)a.ds + slot * (kTile * kTile * 2) + (uint32_t)__builtin_amdgcn_readfirstlane((q_first & (kTile - 1)) * 2);
+    const uint32_t qsb = (uint32_t)(a.q.stride_s * 2), gsb = (uint32_t)(a.dout.stride_s * 2);  // row strides in bytes
+    // a whole tile at once (the first step of an item, and a block this wave skips)
+    auto burst = [&](const void* src, uint32_t dst, uint32_t stride_bytes, int last_row, bool with_last) {
+#pragma unroll
+        for (int p = 0; p < kPaced; ++p) global_to_lds_run_rc(src, sq.rc[p], stride_bytes, last_row, dst + (w + p * NW) * 1024);
+        if (with_last) global_to_lds_run_rc(src, rc_last, stride_bytes, last_row, dst + (SQ::NL - 1) * 1024);
     };
+    // per-row lse / delta / document id of a step: loaded for the step after the current one, written
+    // to LDS when that step begins by wave 1 (lse), wave 2 (delta) and wave 3 (ids).  Every wave issues
+    // both loads, each from the array it is in charge of (no branch: a conditional load would be waited
+    // for on the spot, to merge its result with the value carried otherwise).
+    float row_f = 0.f;
+    int64_t row_d = 0;
+    auto load_rows = [&](uint64_t lse_at, uint64_t delta_at, int r0) {
+        const int li = min(lane, S - 1 - r0);
+        const MA_GLB float* fsrc = (const MA_GLB float*)(w == 2 ? delta_at : lse_at);
+        row_f = fsrc[li];
+        if (HAS_DOC) row_d = ((const MA_GLB int64_t*)drow)[r0 + li];
+    };
+    // the step the loop stands on, and the one after it
+    uint32_t nflags = 0;
+    uint64_t ds_at = 0, nds_at = 0, nq_at = 0, ng_at = 0;
+    // (the fields of the current step's word are carried as variables of their own: decoded from the word
+    // inside the loop, the compiler splits the accumulators' live ranges around the skipped-block path
+    // and spills them)
+    int q0 = 0;
+    bool partial = false, act0 = false, act1 = false;
+    auto decode = [&](uint32_t word) {
+        q0 = (int)(word & 0xffffffu);
+        partial = (word >> 31) != 0;
+        act0 = (word >> 30) & 1u;
+        act1 = (word >> 29) & 1u;
+    };
+    bool have = st.advance(j, hk, b, w);
+    if (have) {
+        MA_LDS uint32_t* rec = st.tab + st.pos * kDkvRecWords;
+        const u32x4 x0 = *(MA_LDS u32x4*)rec, x1 = *(MA_LDS u32x4*)(rec + 4), x2 = *(MA_LDS u32x4*)(rec + 8);
+        const uint32_t flags = __builtin_amdgcn_readfirstlane(x0[0]);
+        nq_at = uniform64(x0[2], x0[3]);
+        ng_at = uniform64(x1[0], x1[1]);
+        ds_at = uniform64(x2[2], x2[3]);
+        decode(flags);
+        const int r0 = q0;
+        const int last = min(BM, S - r0) - 1;
+        burst((const void*)nq_at, lds_addr(Qbuf(0)), qsb, last, w == 0);
+        burst((const void*)ng_at, lds_addr(Gbuf(0)), gsb, last, w == 1);
+        load_rows(uniform64(x1[2], x1[3]), uniform64(x2[0], x2[1]), r0);
+    }
     const uint32_t ds_lane = (uint32_t)((32 * w + r) * (kTile * 2) + 16 * hh);
 
     for (int n = 0; have; ++n) {
+        MA_TICK(0);
         const int cur = n & 1;
         const lds_ptr Qs = Qbuf(cur), Gs = Gbuf(cur);
         MA_LDS float* lse2s = Lbuf(cur);
         MA_LDS float* dls = Ebuf(cur);
         MA_LDS int64_t* qdoc = Dbuf(cur);
-        if (tid < BM) {
-            lse2s[tid] = lse_next * kLog2e;
-            dls[tid] = dl_next;
-            if (HAS_DOC) qdoc[tid] = qd_next;
+        if (w == 1) lse2s[lane] = row_f * kLog2e;
+        if (w == 2) dls[lane] = row_f;
+        if (HAS_DOC && w == 3) qdoc[lane] = row_d;
+        const bool have_next = st.advance(j, hk, b, w);
+        u32x4 x0 = {0, 0, 0, 0}, x1 = x0, x2 = x0;
+        if (have_next) {  // the record of the next step: read now, picked up behind the barrier
+            MA_LDS uint32_t* rec = st.tab + st.pos * kDkvRecWords;
+            x0 = *(MA_LDS u32x4*)rec;
+            x1 = *(MA_LDS u32x4*)(rec + 4);
+            x2 = *(MA_LDS u32x4*)(rec + 8);
         }
         wait_vmem();
         __syncthreads();
+        MA_TICK(1);
 
         const int cq0 = q0;
         const bool cpartial = partial;
         const bool skip[BM / 32] = {!act0, !act1};  // blocks in which this wave has nothing to do
-        char* ds_out = WRITE_DS ? ds_step(hk * G + rep, cq0, tslot) : nullptr;
-        have = st.next();
-        // The tile loads of the next step are spread over this step's first MFMA chains, one run
-        // every few MFMAs (Q tile in the first 32-row block, dO tile in the second): issued in one
-        // burst they fill the memory pipeline and stall the wave with the matrix cores idle.  A
-        // ragged last tile, or a block that is skipped, issues its tile at once.
-        int pace = 0;
-        if (have) {
-            q0 = st.r0;
-            rep = st.rep;
-            tslot = st.tile_slot;
-            partial = st.partial;
-            act0 = st.act0;
-            act1 = st.act1;
-            locate();
-            issue_rows();
-            const bool spread = (q0 + BM <= a.S) & !skip[0] & !skip[1];
-            pace = __builtin_amdgcn_readfirstlane(spread ? my_runs : 0);
-            if (!pace) {
-                issue_q(cur ^ 1);
-                issue_g(cur ^ 1);
-            }
+        MA_GLB char* ds_out = (MA_GLB char*)ds_at;  // (a global pointer: a generic one would make the stores flat ones, counted with the LDS reads)
+        // The tile loads of the next step are spread over the chains of this step's first 32-row block,
+        // one run every four MFMAs (Q tile from the S / dP chain, dO tile from the dV / dK chain): issued
+        // in one burst they fill the memory pipeline and stall the wave with the matrix cores idle, and
+        // issued later in the step they have not landed when the next step begins.
+        int nlast = min(BM, S - cq0) - 1;
+        if (have_next) {
+            nflags = __builtin_amdgcn_readfirstlane(x0[0]);
+            nq_at = uniform64(x0[2], x0[3]);
+            ng_at = uniform64(x1[0], x1[1]);
+            nds_at = uniform64(x2[2], x2[3]);
+            const int nr0 = (int)(nflags & 0xffffffu);
+            nlast = min(BM, S - nr0) - 1;
+            load_rows(uniform64(x1[2], x1[3]), uniform64(x2[0], x2[1]), nr0);
+            if (w == 0) global_to_lds_run_rc((const void*)nq_at, rc_last, qsb, nlast, lds_addr(Qbuf(cur ^ 1)) + (SQ::NL - 1) * 1024);
+            if (w == 1) global_to_lds_run_rc((const void*)ng_at, rc_last, gsb, nlast, lds_addr(Gbuf(cur ^ 1)) + (SQ::NL - 1) * 1024);
         }
         const uint32_t qdst = lds_addr(Qbuf(cur ^ 1)), gdst = lds_addr(Gbuf(cur ^ 1));
 
-#pragma unroll 1
-        for (int mb = 0; mb < BM / 32; ++mb) {
+        // The two 32-row blocks of the step are two copies of the same code (mb is a compile-time
+        // constant in each), so that each chain carries exactly the loads planned for it.
+        auto block = [&](auto mb_c) {
+            constexpr int mb = decltype(mb_c)::value;
+            MA_TICK(2);
             const int qb0 = cq0 + 32 * mb;
-            if (mb ? skip[1] : skip[0]) {
+            // which runs of which tile (0: Q, 1: dO) the block's two chains move: {tile, first run, runs}
+            constexpr int kPlanA[3] = {kDkvPlan[mb][0][0], kDkvPlan[mb][0][1] * kPaced / 8, kDkvPlan[mb][0][2] * kPaced / 8};
+            constexpr int kPlanB[3] = {kDkvPlan[mb][1][0], kDkvPlan[mb][1][1] * kPaced / 8, kDkvPlan[mb][1][2] * kPaced / 8};
+            auto move_run = [&](auto tile_c, auto run_c) {
+                constexpr int run = decltype(run_c)::value;
+                if constexpr (decltype(tile_c)::value == 0)
+                    global_to_lds_run_rc((const void*)nq_at, sq.rc[run], qsb, nlast, qdst + w * 1024 + run * (NW * 1024));
+                else
+                    global_to_lds_run_rc((const void*)ng_at, sq.rc[run], gsb, nlast, gdst + w * 1024 + run * (NW * 1024));
+            };
+            if (skip[mb]) {
                 if (WRITE_DS) {
 #pragma unroll
-                    for (int pr = 0; pr < 2; ++pr) *(u32x4*)(ds_out + ds_lane + 64 * mb + 32 * pr) = u32x4{0, 0, 0, 0};
+                    for (int pr = 0; pr < 2; ++pr) *(MA_GLB u32x4*)(ds_out + ds_lane + 64 * mb + 32 * pr) = u32x4{0, 0, 0, 0};
                 }
-                continue;
+                if (have_next) {  // the loads its chains would have carried
+                    static_for<0, kPlanA[2]>([&](auto r) { move_run(std::integral_constant<int, kPlanA[0]>{}, std::integral_constant<int, kPlanA[1] + decltype(r)::value>{}); });
+                    static_for<0, kPlanB[2]>([&](auto r) { move_run(std::integral_constant<int, kPlanB[0]>{}, std::integral_constant<int, kPlanB[1] + decltype(r)::value>{}); });
+                }
+                return;
             }
-            const __bf16* psrc = (const __bf16*)(mb ? gsrc : qsrc);
-            const uint32_t pdst = mb ? gdst : qdst, psb = mb ? gsb : qsb;
-            constexpr int kEvery = (2 * KK) / decltype(sq)::PER;
-            static_assert(kEvery >= 1, "pacing");
-            auto pace_hook = [&](auto idx) {
+            auto a_hook = [&](auto idx) {
                 constexpr int i = decltype(idx)::value;
-                if constexpr (i % kEvery == kEvery - 1) sq.template issue_one<i / kEvery>(psrc, pdst, w, pace, psb);
+                if constexpr (kPlanA[2] > 0) {
+                    constexpr int every = (2 * KK) / kPlanA[2];
+                    if constexpr (i % every == every - 1) move_run(std::integral_constant<int, kPlanA[0]>{}, std::integral_constant<int, kPlanA[1] + i / every>{});
+                }
+            };
+            auto b_hook = [&](auto idx) {
+                constexpr int i = decltype(idx)::value;
+                if constexpr (kPlanB[2] > 0) {
+                    constexpr int every = (2 * KK) / kPlanB[2];
+                    if constexpr (i % every == every - 1) move_run(std::integral_constant<int, kPlanB[0]>{}, std::integral_constant<int, kPlanB[1] + i / every>{});
+                }
             };
 
             // S = Q K^T and dP = dO V^T for 32 q rows x the wave's 32 kv rows (lane owns one kv row)
             f32x16 s, dp;
             const uint32_t roff = (uint32_t)(32 * mb * TL::kPitch);
-            rowfrag_gemm2<D, kBPipe, false, false>(lds_addr(Qs) + rbase + roff, kf, s, lds_addr(Gs) + rbase + roff, vf, dp, pace_hook);
+            rowfrag_gemm2<D, kBPipe, false, false>(lds_addr(Qs) + rbase + roff, kf, s, lds_addr(Gs) + rbase + roff, vf, dp, a_hook);
+            MA_TICK(3);
 
             bf16x8 pf[2], dsf[2];
             // d = q - kv for element v is drel + 8*(v/4) + v%4; range test as one unsigned compare
             const int drel = qb0 + 4 * hh - kv;
             const int dlo = bounded ? 0 : -0x40000000;
-            const int dhi = min(wlim, a.S - 1 - kv);              // q - kv <= window, q < S
+            const int dhi = min(wlim, S - 1 - kv);              // q - kv <= window, q < S
             const unsigned span = (unsigned)(dhi - dlo);
             const bool some = (dhi >= dlo) & kvalid;
             const unsigned t0 = (unsigned)(drel - dlo);
@@ -339,15 +505,24 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
                     const u32x4 f = __builtin_bit_cast(u32x4, dsf[pr]);   // dwords 0,1: g4 = 2*pr, dwords 2,3: g4 = 2*pr + 1
                     const auto s0 = __builtin_amdgcn_permlane32_swap(f[0], f[2], false, false);
                     const auto s1 = __builtin_amdgcn_permlane32_swap(f[1], f[3], false, false);
-                    *(u32x4*)(ds_out + ds_lane + 64 * mb + 32 * pr) = u32x4{s0[0], s1[0], s0[1], s1[1]};
+                    *(MA_GLB u32x4*)(ds_out + ds_lane + 64 * mb + 32 * pr) = u32x4{s0[0], s1[0], s0[1], s1[1]};
                 }
             }
             // dV^T += dO^T P and dK^T += Q^T dS  (accumulators stay in AGPRs)
             // (one read pipeline for both products: it is filled once, and one fence serves both)
-            trfrag_gemm_two<D, 2, kBPipe>(lds_addr(Gs) + tbase + roff, pf, dvacc, lds_addr(Qs) + tbase + roff, dsf, dkacc);
-        }
+            MA_TICK(4);
+            trfrag_gemm_two<D, 2, kBPipe>(lds_addr(Gs) + tbase + roff, pf, dvacc, lds_addr(Qs) + tbase + roff, dsf, dkacc, b_hook);
+            MA_TICK(5);
+        };
+        block(std::integral_constant<int, 0>{});
+        block(std::integral_constant<int, 1>{});
+        MA_TICK(6);
+        decode(nflags);
+        ds_at = nds_at;
+        have = have_next;
     }
 
+    wait_vmem();      // (the chains of the last step have fetched its own tiles once more: no test in the hooks)
     __syncthreads();  // everyone is done with the tiles: reuse the ring as store scratch
     mfma_fence();
     {
@@ -355,8 +530,8 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
         const lds_ptr scratch = lds0 + w * 32 * kPitchO;
         __bf16* okp = (__bf16*)a.dk.ptr + b * a.dk.stride_b + hk * a.dk.stride_h;
         __bf16* ovp = (__bf16*)a.dv.ptr + b * a.dv.stride_b + hk * a.dv.stride_h;
-        store_tile_T<D>(scratch, dkacc, a.scale, okp, a.dk.stride_s, kw_lo, a.S, lane);
-        store_tile_T<D>(scratch, dvacc, 1.0f, ovp, a.dv.stride_s, kw_lo, a.S, lane);
+        store_tile_T<D>(scratch, dkacc, a.scale, okp, a.dk.stride_s, kw_lo, S, lane);
+        store_tile_T<D>(scratch, dvacc, 1.0f, ovp, a.dv.stride_s, kw_lo, S, lane);
     }
 }
 
@@ -368,10 +543,27 @@ __global__ __launch_bounds__(kBwdThreads, D <= 128 ? MA_DKV_WAVES : 1) void attn
     MA_LDS int* box = (MA_LDS int*)((lds_ptr)smem_raw + (4 * Tile<D>::bytes(kStep) + 2 * kStep * (4 + 4 + 8)));
     WorkQueue wq;
     wq.init(a.map.work_counters, kQueueDkv, work_grid(a.B * a.T, a.Hkv, 1));
+#ifdef MA_TICKS
+    Ticks ticks;
+    const unsigned long long t_start = __builtin_readcyclecounter();
+    for (int id = wq.next(box); id >= 0; id = wq.next(box)) {
+        MA_TICK(7);
+        attn_bwd_dkv_bf16_item<D, HAS_DOC, WRITE_DS>(fresh_args(), id, ticks);
+        __syncthreads();
+        MA_TICK(8);
+    }
+    if (threadIdx.x == MA_T_WAVE * 64) {
+        atomicAdd(&ma_dbg_ticks[0], ticks.acc);
+        atomicAdd(&ma_dbg_ticks[1], (unsigned long long)ticks.n);
+        atomicAdd(&ma_dbg_ticks[2], __builtin_readcyclecounter() - t_start);
+        atomicAdd(&ma_dbg_ticks[3], 1ull);
+    }
+#else
     for (int id = wq.next(box); id >= 0; id = wq.next(box)) {
         attn_bwd_dkv_bf16_item<D, HAS_DOC, WRITE_DS>(fresh_args(), id);
         __syncthreads();  // the item's LDS (and the box) are free again
     }
+#endif
     wq.leave();
 }
 
@@ -907,7 +1099,7 @@ static int bwd_dd(const AttnArgs& a, hipStream_t st) {
         rc = check_launch("attn_delta_bf16_kernel");
         if (rc) return rc;
     }
-    const size_t lds_kv = (size_t)4 * Tile<D>::bytes(kStep) + 2 * kStep * (4 + 4 + 8) + 16 + (kBwdThreads / 64) * 512;  // + work-queue box, step tables
+    const size_t lds_kv = (size_t)4 * Tile<D>::bytes(kStep) + 2 * kStep * (4 + 4 + 8) + 16 + (kBwdThreads / 64) * kDkvRecBytes;  // + work-queue box, step records
     if (hand_over) {
         if (a.stages & MA_BWD_DKV) {
             rc = opt_in_lds(attn_bwd_dkv_bf16_kernel<D, HAS_DOC, true>, lds_kv, "attn_bwd_dkv_bf16");
@@ -973,3 +1165,10 @@ int launch_attn_bwd_bf16(const AttnArgs& a, hipStream_t st) {
 }
 
 }  // namespace ma
+
+#ifdef MA_TICKS
+extern "C" void ma_dbg_read_ticks(unsigned long long* out, int reset) {
+    (void)hipMemcpyFromSymbol(out, HIP_SYMBOL(ma::ma_dbg_ticks), sizeof(unsigned long long) * 4);
+    if (reset) { unsigned long long z[4] = {0, 0, 0, 0}; (void)hipMemcpyToSymbol(HIP_SYMBOL(ma::ma_dbg_ticks), z, sizeof(z)); }
+}
+#endif
