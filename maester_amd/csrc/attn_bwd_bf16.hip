@@ -151,8 +151,13 @@ struct DkvSteps {
         const int lane = __lane_id();
         const int G = a.Hq / a.Hkv;
         const size_t mrow = (size_t)b * a.T + j;
+        const bool use_rng = HAS_DOC && a.map.block_doc_range != nullptr;
+        const int64_t* rng = use_rng ? a.map.block_doc_range + (size_t)b * (2 * ((a.S + 63) / 64)) * 2 : nullptr;
+        DocRange own;  // id range of the wave's own kv rows: in the same round trip as the list lengths
         int np, nf;
-        scalar_load2(a.map.q_num_blocks + mrow, a.map.full_q_num_blocks + mrow, np, nf);
+        if (use_rng) scalar_load2_range(a.map.q_num_blocks + mrow, a.map.full_q_num_blocks + mrow,
+                                        rng + (size_t)(min(j * kTile + 32 * w, a.S - 1) / MA_DOC_BLOCK) * 2, np, nf, own);
+        else scalar_load2(a.map.q_num_blocks + mrow, a.map.full_q_num_blocks + mrow, np, nf);
         const int n = np + nf, per_pass = n * (kTile / kStep), total = per_pass * G;
         const bool bounded = a.causal || a.window >= 0, windowed = a.window >= 0;
         const int wlim = windowed ? (int)min(a.window, (int64_t)0x3fffffff) : 0x7fffffff;
@@ -160,13 +165,8 @@ struct DkvSteps {
         int vis_lo, vis_hi, blk_lo, blk_hi;
         visibility_limits(true, j * kTile, j * kTile + kTile - 1, kStep, bounded, wlim, windowed, vis_lo, vis_hi);
         visibility_limits(true, kw_lo, kw_hi, 32, bounded, wlim, windowed, blk_lo, blk_hi);
-        const bool use_rng = HAS_DOC && a.map.block_doc_range != nullptr;
-        const int64_t* rng = use_rng ? a.map.block_doc_range + (size_t)b * (2 * ((a.S + 63) / 64)) * 2 : nullptr;
         int64_t own_lo = 0, own_hi = 0;
         if (use_rng) {
-            DocRange own;
-            own.load(rng + (size_t)(min(kw_lo, a.S - 1) / MA_DOC_BLOCK) * 2);
-            own.ready();
             own_lo = own.lo();
             own_hi = own.hi();
         }
@@ -261,6 +261,7 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
     const bool kvalid = kv < a.S;
     const bool bounded = a.causal || a.window >= 0;
     const float sl2 = a.scale * kLog2e;
+    const float neg_inv_scale = -1.0f / a.scale;
     const int S = a.S;
 
     const __bf16* kp = (const __bf16*)a.k.ptr + b * a.k.stride_b + hk * a.k.stride_h;
@@ -370,8 +371,8 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
         MA_LDS float* lse2s = Lbuf(cur);
         MA_LDS float* dls = Ebuf(cur);
         MA_LDS int64_t* qdoc = Dbuf(cur);
-        if (w == 1) lse2s[lane] = row_f * kLog2e;
-        if (w == 2) dls[lane] = row_f;
+        if (w == 1) lse2s[lane] = row_f * neg_inv_scale;  // -lse / scale: the addend of S
+        if (w == 2) dls[lane] = -row_f;                    // -delta: the addend of dP
         if (HAS_DOC && w == 3) qdoc[lane] = row_d;
         const bool have_next = st.advance(j, hk, b, w);
         u32x4 x0 = {0, 0, 0, 0}, x1 = x0, x2 = x0;
@@ -450,9 +451,22 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
             };
 
             // S = Q K^T and dP = dO V^T for 32 q rows x the wave's 32 kv rows (lane owns one kv row)
+            // The accumulators start from -lse / scale and -delta of their q rows (an element's row is
+            // 8 * (v / 4) + 4 * hh + v % 4), read from LDS straight into them: the chain then leaves
+            // S - lse / scale and dP - delta, and neither is touched by the vector ALU for it.
             f32x16 s, dp;
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                const f32x4 l4 = *(MA_LDS f32x4*)(lse2s + 32 * mb + 8 * g4 + 4 * hh);
+                const f32x4 e4 = *(MA_LDS f32x4*)(dls + 32 * mb + 8 * g4 + 4 * hh);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    s[4 * g4 + e] = l4[e];
+                    dp[4 * g4 + e] = e4[e];
+                }
+            }
             const uint32_t roff = (uint32_t)(32 * mb * TL::kPitch);
-            rowfrag_gemm2<D, kBPipe, false, false>(lds_addr(Qs) + rbase + roff, kf, s, lds_addr(Gs) + rbase + roff, vf, dp, a_hook);
+            rowfrag_gemm2<D, kBPipe, false, false, decltype(a_hook)&, false, true>(lds_addr(Qs) + rbase + roff, kf, s, lds_addr(Gs) + rbase + roff, vf, dp, a_hook);
             MA_TICK(3);
 
             bf16x8 pf[2], dsf[2];
@@ -470,8 +484,6 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
 #pragma unroll
                 for (int g4 = 0; g4 < 4; ++g4) {
                     const int qoff = 32 * mb + 8 * g4 + 4 * hh;
-                    const f32x4 l4 = *(MA_LDS f32x4*)(lse2s + qoff);
-                    const f32x4 e4 = *(MA_LDS f32x4*)(dls + qoff);
                     i64x2 ida = {0, 0}, idb = {0, 0};
                     if (HAS_DOC && MASKED) {
                         ida = *(MA_LDS i64x2*)(qdoc + qoff);
@@ -481,13 +493,13 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         const int v = 4 * g4 + e;
-                        float p = fast_exp2(s[v] * sl2 - l4[e]);
+                        float p = fast_exp2(s[v] * sl2);
                         if (MASKED) {
                             bool ok = (t0 + (unsigned)(8 * g4 + e) <= span) & some;
                             if (HAS_DOC) ok = ok & (ids[e] == dock);
                             p = ok ? p : 0.f;
                         }
-                        const float ds = p * (dp[v] - e4[e]);
+                        const float ds = p * dp[v];
                         pf[v >> 3][v & 7] = (__bf16)p;
                         dsf[v >> 3][v & 7] = (__bf16)ds;
                     }

@@ -25,6 +25,26 @@
 
 namespace ma {
 
+#ifdef MA_TICKS
+// debug build only: cycles a wave spends between two marked points of the kernel
+__device__ unsigned long long ma_dbg_ticks_fwd[4];
+struct TicksF {
+    unsigned long long begin = 0, acc = 0;
+    unsigned n = 0;
+    bool armed = false;
+    template <int ID>
+    __device__ __forceinline__ void at() {
+        if constexpr (ID == MA_T_END) {
+            if (armed) { acc += __builtin_readcyclecounter() - begin; ++n; armed = false; }
+        }
+        if constexpr (ID == MA_T_BEGIN) { begin = __builtin_readcyclecounter(); armed = true; }
+    }
+};
+#define MA_TICK(id) ticks.template at<id>()
+#else
+#define MA_TICK(id)
+#endif
+
 constexpr int kPairThreads = 256;
 constexpr int kPairBN = 64;   // kv rows staged per step
 #ifndef MA_PAIR_PK
@@ -35,7 +55,11 @@ constexpr int kPairPipeK = MA_PAIR_PK;  // LDS fragment reads in flight ahead of
 constexpr int kPairPipeV = MA_PAIR_PV;
 
 template <int D, bool HAS_DOC>
-__device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int wg_id) {
+__device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int wg_id
+#ifdef MA_TICKS
+    , TicksF& ticks
+#endif
+) {
     using TL = Tile<D>;
     constexpr int KK = D / 16;
     constexpr int DB = D / 32;
@@ -80,10 +104,6 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
     const bool use_rng = HAS_DOC && a.map.block_doc_range != nullptr;
     const int64_t* rng_row = use_rng ? a.map.block_doc_range + (size_t)b * (2 * ((a.S + 63) / 64)) * 2 : nullptr;
     DocRange own;
-    if (use_rng) {
-        own.load(rng_row + (size_t)(min(qw_lo, a.S - 1) / MA_DOC_BLOCK) * 2);
-        own.ready();
-    }
 
     DirectStager<D, BN, NW> sk;
     sk.init(w, lane);
@@ -102,7 +122,10 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
         int lo, hi;
         visibility_limits(false, i * kTile, i * kTile + kTile - 1, BN, bounded, wlim, windowed, lo, hi);
         int n_partial, n_full;
-        scalar_load2(a.map.kv_num_blocks + mrow, a.map.full_kv_num_blocks + mrow, n_partial, n_full);
+        // (the id range of the wave's own rows comes in the same round trip as the list lengths)
+        if (use_rng) scalar_load2_range(a.map.kv_num_blocks + mrow, a.map.full_kv_num_blocks + mrow,
+                                        rng_row + (size_t)(min(qw_lo, a.S - 1) / MA_DOC_BLOCK) * 2, n_partial, n_full, own);
+        else scalar_load2(a.map.kv_num_blocks + mrow, a.map.full_kv_num_blocks + mrow, n_partial, n_full);
         st.init(a.map.kv_indices + mrow * a.T, n_partial, a.map.full_kv_indices + mrow * a.T, n_full, 1, false, a.S, lo, hi,
                 blk_lo, blk_hi, use_rng ? rng_row : nullptr, use_rng ? own.lo() : 0, use_rng ? own.hi() : 0, steps_slot);
         st.prime();
@@ -154,12 +177,14 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
     }
 
     for (int n = 0; have; ++n) {
+        MA_TICK(0);
         const int cur = n & 1;
         const lds_ptr Ks = Kbuf(cur), Vs = Vbuf(cur);
         MA_LDS int64_t* kdoc = Dbuf(cur);
         if (HAS_DOC && partial && tid < BN) kdoc[tid] = kd_next;
         wait_vmem();
         __syncthreads();
+        MA_TICK(1);
 
         const int ck0 = k0;
         const bool cpartial = partial;
@@ -196,6 +221,7 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
 
 #pragma unroll 1
         for (int nb = 0; nb < 2; ++nb) {
+            MA_TICK(2);
             if (!(nb ? act[1] : act[0])) continue;
             const int lim = nb == first ? pace : 0;
             constexpr int kEvery = (2 * KK) / decltype(sk)::PER;  // both chains have 2*KK MFMAs
@@ -213,6 +239,7 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
             // S^T of both heads for 32 kv rows (lane owns one q row, 16 of the kv rows)
             f32x16 sa, sb;
             rowfrag_gemm_dual<D, kPairPipeK>(lds_addr(Ks) + rbase + roff, qa, qb, sa, sb, pace_k);
+            MA_TICK(3);
 
             // mask (shared by the two heads) and row maxima on the unscaled scores
             float mxa = -INFINITY, mxb = -INFINITY;
@@ -274,8 +301,11 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
             lb += rsb + xor32(rsb);
 
             // O^T += V^T P^T for both heads: every transposed V fragment feeds two MFMAs
+            MA_TICK(4);
             trfrag_gemm_dual<D, 2, kPairPipeV>(lds_addr(Vs) + tbase + roff, pa, pb, oa, ob, pace_v);
+            MA_TICK(5);
         }
+        MA_TICK(6);
     }
 
     __syncthreads();  // every wave is done with the K/V buffers, and with the flag
@@ -329,10 +359,27 @@ __global__ __launch_bounds__(kPairThreads) void attn_fwd_pair_bf16_kernel(AttnAr
     MA_LDS int* box = (MA_LDS int*)((lds_ptr)smem_raw + (4 * Tile<D>::bytes(kPairBN) + 2 * kPairBN * 8 + 4));
     WorkQueue wq;
     wq.init(a.map.work_counters, kQueueFwd, work_grid(a.B * a.T, a.Hkv, a.Hq / a.Hkv / 2));
+#ifdef MA_TICKS
+    TicksF ticks;
+    const unsigned long long t_start = __builtin_readcyclecounter();
+    for (int id = wq.next(box); id >= 0; id = wq.next(box)) {
+        MA_TICK(7);
+        attn_fwd_pair_bf16_item<D, HAS_DOC>(fresh_args(), id, ticks);
+        __syncthreads();
+        MA_TICK(8);
+    }
+    if (threadIdx.x == MA_T_WAVE * 64) {
+        atomicAdd(&ma_dbg_ticks_fwd[0], ticks.acc);
+        atomicAdd(&ma_dbg_ticks_fwd[1], (unsigned long long)ticks.n);
+        atomicAdd(&ma_dbg_ticks_fwd[2], __builtin_readcyclecounter() - t_start);
+        atomicAdd(&ma_dbg_ticks_fwd[3], 1ull);
+    }
+#else
     for (int id = wq.next(box); id >= 0; id = wq.next(box)) {
         attn_fwd_pair_bf16_item<D, HAS_DOC>(fresh_args(), id);
         __syncthreads();  // the item's LDS (and the box) are free again
     }
+#endif
     wq.leave();
 }
 
@@ -362,3 +409,10 @@ int launch_attn_fwd_pair_bf16(const AttnArgs& a, hipStream_t st) {
 }
 
 }  // namespace ma
+
+#ifdef MA_TICKS
+extern "C" void ma_dbg_read_ticks_fwd(unsigned long long* out, int reset) {
+    (void)hipMemcpyFromSymbol(out, HIP_SYMBOL(ma::ma_dbg_ticks_fwd), sizeof(unsigned long long) * 4);
+    if (reset) { unsigned long long z[4] = {0, 0, 0, 0}; (void)hipMemcpyToSymbol(HIP_SYMBOL(ma::ma_dbg_ticks_fwd), z, sizeof(z)); }
+}
+#endif

@@ -459,6 +459,13 @@ struct DocRange {      // one block
     __device__ __forceinline__ int64_t lo() const { return (int64_t)(((uint64_t)(uint32_t)raw[1] << 32) | (uint32_t)raw[0]); }
     __device__ __forceinline__ int64_t hi() const { return (int64_t)(((uint64_t)(uint32_t)raw[3] << 32) | (uint32_t)raw[2]); }
 };
+// two list lengths and one block's id range in one round trip: the three loads and their wait are one
+// asm statement (a load left in flight across other code could land in registers the compiler has
+// meanwhile given to something else)
+__device__ __forceinline__ void scalar_load2_range(const int32_t* p, const int32_t* q, const int64_t* entry, int& a, int& b, DocRange& r) {
+    asm volatile("s_load_dword %0, %3, 0x0\n\ts_load_dword %1, %4, 0x0\n\ts_load_dwordx4 %2, %5, 0x0\n\ts_waitcnt lgkmcnt(0)"
+                 : "=&s"(a), "=&s"(b), "=&s"(r.raw) : "s"(p), "s"(q), "s"(entry) : "memory");
+}
 struct DocRange2 {     // two consecutive blocks (one 64-row step)
     i32x8_t raw;
     __device__ __forceinline__ void load(const int64_t* entry) { asm volatile("s_load_dwordx8 %0, %1, 0x0" : "=s"(raw) : "s"(entry)); }

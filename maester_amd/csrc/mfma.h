@@ -243,7 +243,8 @@ __device__ __forceinline__ void rowfrag_gemm(uint32_t row_addr, const bf16x8* re
 // SEQ = false interleaves them MFMA by MFMA; SEQ = true finishes acc0 (MFMAs 0..KK-1) before acc1
 // (MFMAs KK..2KK-1), so that hooks of the second half can already work on acc0 with the vector ALU
 // (from MFMA KK+1 on: the result of an MFMA is readable two MFMAs later).
-template <int D, int P, bool SWAP = false, bool REG_A = true, typename Hook = NoHook, bool SEQ = false>
+// PRESET: the accumulators come in holding the addends of the two products instead of being overwritten.
+template <int D, int P, bool SWAP = false, bool REG_A = true, typename Hook = NoHook, bool SEQ = false, bool PRESET = false>
 __device__ __forceinline__ void rowfrag_gemm2(uint32_t row_addr0, const bf16x8* reg0, f32x16& acc0, uint32_t row_addr1,
                                               const bf16x8* reg1, f32x16& acc1, Hook&& hook = Hook{}) {
     constexpr int KK = D / 16;
@@ -262,7 +263,7 @@ __device__ __forceinline__ void rowfrag_gemm2(uint32_t row_addr0, const bf16x8* 
         // the register fragment is handed to the asm statement as it is (no copy: a copy of an
         // AGPR-resident fragment would need AGPRs of its own)
         auto one = [&](f32x16& acc, const bf16x8& rg) {
-            if constexpr (kk == 0) {
+            if constexpr (kk == 0 && !PRESET) {
                 if constexpr (!REG_A) { if constexpr (SWAP) mfma32_vv_zero(acc, rg, t[i]); else mfma32_vv_zero(acc, t[i], rg); }
                 else if constexpr (SWAP) mfma32_av_zero(acc, rg, t[i]);
                 else mfma32_va_zero(acc, t[i], rg);
