@@ -53,6 +53,21 @@ constexpr int kPairBN = 64;   // kv rows staged per step
 #endif
 constexpr int kPairPipeK = MA_PAIR_PK;  // LDS fragment reads in flight ahead of the MFMAs (registers are tight)
 constexpr int kPairPipeV = MA_PAIR_PV;
+// Which chain of a step carries which of the next step's tile loads, in eighths of a wave's runs:
+// kPairPlan[block][chain (0: S^T, 1: O^T)] = {tile (0: K, 1: V), first eighth, eighths}.  K rides in S^T
+// chains only (the pass that only finds row maxima has no O^T chains, and needs no V).
+#ifndef MA_PAIR_PLACE
+#define MA_PAIR_PLACE 1
+#endif
+#if MA_PAIR_PLACE == 0
+constexpr int kPairPlan[2][2][3] = {{{0, 0, 8}, {1, 0, 8}}, {{0, 0, 0}, {0, 0, 0}}};
+#elif MA_PAIR_PLACE == 1
+constexpr int kPairPlan[2][2][3] = {{{0, 0, 8}, {0, 0, 0}}, {{1, 0, 8}, {0, 0, 0}}};
+#elif MA_PAIR_PLACE == 2
+constexpr int kPairPlan[2][2][3] = {{{0, 0, 8}, {1, 0, 4}}, {{1, 4, 4}, {0, 0, 0}}};
+#elif MA_PAIR_PLACE == 3
+constexpr int kPairPlan[2][2][3] = {{{0, 0, 8}, {0, 0, 0}}, {{0, 0, 0}, {1, 0, 8}}};
+#endif
 
 template <int D, bool HAS_DOC>
 __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int wg_id
@@ -105,9 +120,20 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
     const int64_t* rng_row = use_rng ? a.map.block_doc_range + (size_t)b * (2 * ((a.S + 63) / 64)) * 2 : nullptr;
     DocRange own;
 
-    DirectStager<D, BN, NW> sk;
+    // The K and V tiles have the same shape: one set of slots.  Every wave moves the same number of runs
+    // of a tile from inside its MFMA chains (kPaced); the run that is left over (a tile is 4 * kPaced + 1
+    // runs) is moved by wave 0 (K) or wave 1 (V) when the step begins.
+    using SK = DirectStager<D, BN, NW>;
+    constexpr int kPaced = (SK::NL - 1) / NW;
+    static_assert(SK::NL == NW * kPaced + 1 && (2 * KK) % kPaced == 0 && 4 * DB == 2 * KK, "tile runs per wave");
+    SK sk;
     sk.init(w, lane);
-    const int my_runs = decltype(sk)::runs_of(w);
+    uint32_t rc_last;  // the left-over run, whichever wave moves it
+    {
+        int row, chunk;
+        SK::slot(SK::NL - 1, lane, row, chunk);
+        rc_last = (uint32_t)(row << 16 | chunk * 16);
+    }
     int64_t kd_next = 0;
 
     // The walk over the kv tiles: its index loads go out first, then both heads' Q rows, which go
@@ -117,6 +143,7 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
     bool have;
     int k0;
     bool partial, act0, act1;  // of the step the walk stands on: tile kind, blocks this wave has work in
+    const char *ksrc = kp, *vsrc = vp;  // its K and V rows
     MA_LDS uint32_t* steps_slot = (MA_LDS uint32_t*)(lds0 + 4 * TL::bytes(BN) + 2 * BN * 8 + 16) + w * 64;
     auto walk_init = [&]() {
         int lo, hi;
@@ -138,8 +165,10 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
         act1 = st.act1;
         if (have) {
             const int rows_valid = min(BN, a.S - k0);
-            sk.issue((const __bf16*)(kp + (uint64_t)(uint32_t)k0 * ksb), Kbuf(0), w, lane, rows_valid, a.k.stride_s);
-            sk.issue((const __bf16*)(vp + (uint64_t)(uint32_t)k0 * vsb), Vbuf(0), w, lane, rows_valid, a.v.stride_s);
+            ksrc = kp + (uint64_t)(uint32_t)k0 * ksb;
+            vsrc = vp + (uint64_t)(uint32_t)k0 * vsb;
+            sk.issue((const __bf16*)ksrc, Kbuf(0), w, lane, rows_valid, a.k.stride_s);
+            sk.issue((const __bf16*)vsrc, Vbuf(0), w, lane, rows_valid, a.v.stride_s);
             if (HAS_DOC && partial && tid < BN) kd_next = drow[min(k0 + tid, a.S - 1)];
         }
     };
@@ -189,13 +218,13 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
         const int ck0 = k0;
         const bool cpartial = partial;
         const bool act[2] = {act0, act1};
-        have = st.next();
-        // the tile loads of the next step ride in the chains of the first active block (K in its S^T
-        // chain, V in its O^T chain); a ragged last tile or a step without chains issues them at once
-        int pace = 0;
-        const char *ksrc = kp, *vsrc = vp;
-        const int first = act[0] ? 0 : 1;
-        if (have) {
+        const bool have_next = st.next();
+        // The tile loads of the next step ride in this step's chains, one run every few MFMAs (see
+        // kPairPlan): issued in one burst they fill the memory pipeline and stall the wave with the
+        // matrix cores idle.  On the last step of a walk the chains fetch the current tiles once more,
+        // into the free half of the ring: cheaper than a test in every hook.
+        int nlast = min(BN, a.S - ck0) - 1;
+        if (have_next) {
             k0 = st.r0;
             partial = st.partial;
             act0 = st.act0;
@@ -203,12 +232,9 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
             ksrc = kp + (uint64_t)(uint32_t)k0 * ksb;
             vsrc = vp + (uint64_t)(uint32_t)k0 * vsb;
             if (HAS_DOC && partial && tid < BN) kd_next = drow[min(k0 + tid, a.S - 1)];
-            pace = __builtin_amdgcn_readfirstlane(((k0 + BN <= a.S) & (act[0] | act[1]) & (mode != 1)) ? my_runs : 0);
-            if (!pace) {
-                const int rows_valid = min(BN, a.S - k0);
-                sk.issue((const __bf16*)ksrc, Kbuf(cur ^ 1), w, lane, rows_valid, a.k.stride_s);
-                sk.issue((const __bf16*)vsrc, Vbuf(cur ^ 1), w, lane, rows_valid, a.v.stride_s);
-            }
+            nlast = min(BN, a.S - k0) - 1;
+            if (w == 0) global_to_lds_run_rc(ksrc, rc_last, ksb, nlast, lds_addr(Kbuf(cur ^ 1)) + (SK::NL - 1) * 1024);
+            if (w == 1 && mode != 1) global_to_lds_run_rc(vsrc, rc_last, vsb, nlast, lds_addr(Vbuf(cur ^ 1)) + (SK::NL - 1) * 1024);
         }
         const uint32_t kdst = lds_addr(Kbuf(cur ^ 1)), vdst = lds_addr(Vbuf(cur ^ 1));
 
@@ -219,26 +245,52 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
         const bool some = wlim >= dlo;
         const unsigned t0 = (unsigned)(qrel - dlo);
 
-#pragma unroll 1
-        for (int nb = 0; nb < 2; ++nb) {
+        // The two 32-row blocks of the step are two copies of the same code (nb is a compile-time
+        // constant in each), so that each chain carries exactly the loads planned for it.
+        auto block = [&](auto nb_c) {
+            constexpr int nb = decltype(nb_c)::value;
             MA_TICK(2);
-            if (!(nb ? act[1] : act[0])) continue;
-            const int lim = nb == first ? pace : 0;
-            constexpr int kEvery = (2 * KK) / decltype(sk)::PER;  // both chains have 2*KK MFMAs
-            static_assert(kEvery >= 1 && 4 * DB == 2 * KK, "pacing");
-            auto pace_k = [&](auto idx) {
-                constexpr int c = decltype(idx)::value;
-                if constexpr (c % kEvery == kEvery - 1) sk.template issue_one<c / kEvery>((const __bf16*)ksrc, kdst, w, lim, ksb);
+            constexpr int kPlanA[3] = {kPairPlan[nb][0][0], kPairPlan[nb][0][1] * kPaced / 8, kPairPlan[nb][0][2] * kPaced / 8};
+            constexpr int kPlanB[3] = {kPairPlan[nb][1][0], kPairPlan[nb][1][1] * kPaced / 8, kPairPlan[nb][1][2] * kPaced / 8};
+            static_assert(kPlanB[2] == 0 || kPlanB[0] == 1, "K rides in S^T chains only");
+            auto move_run = [&](auto tile_c, auto run_c) {
+                constexpr int run = decltype(run_c)::value;
+                if constexpr (decltype(tile_c)::value == 0)
+                    global_to_lds_run_rc(ksrc, sk.rc[run], ksb, nlast, kdst + w * 1024 + run * (NW * 1024));
+                else
+                    global_to_lds_run_rc(vsrc, sk.rc[run], vsb, nlast, vdst + w * 1024 + run * (NW * 1024));
             };
-            auto pace_v = [&](auto idx) {
+            auto burst_plan = [&](auto plan_c) {
+                constexpr int which = decltype(plan_c)::value;
+                constexpr int tile = which ? kPlanB[0] : kPlanA[0], first = which ? kPlanB[1] : kPlanA[1], count = which ? kPlanB[2] : kPlanA[2];
+                static_for<0, count>([&](auto r) { move_run(std::integral_constant<int, tile>{}, std::integral_constant<int, first + decltype(r)::value>{}); });
+            };
+            if (!act[nb]) {
+                if (have_next) {  // the loads its chains would have carried
+                    burst_plan(std::integral_constant<int, 0>{});
+                    if (mode != 1) burst_plan(std::integral_constant<int, 1>{});
+                }
+                return;
+            }
+            auto a_hook = [&](auto idx) {
                 constexpr int c = decltype(idx)::value;
-                if constexpr (c % kEvery == kEvery - 1) sk.template issue_one<c / kEvery>((const __bf16*)vsrc, vdst, w, lim, vsb);
+                if constexpr (kPlanA[2] > 0) {
+                    constexpr int every = (2 * KK) / kPlanA[2];
+                    if constexpr (c % every == every - 1) move_run(std::integral_constant<int, kPlanA[0]>{}, std::integral_constant<int, kPlanA[1] + c / every>{});
+                }
+            };
+            auto b_hook = [&](auto idx) {
+                constexpr int c = decltype(idx)::value;
+                if constexpr (kPlanB[2] > 0) {
+                    constexpr int every = (2 * KK) / kPlanB[2];
+                    if constexpr (c % every == every - 1) move_run(std::integral_constant<int, kPlanB[0]>{}, std::integral_constant<int, kPlanB[1] + c / every>{});
+                }
             };
             const uint32_t roff = (uint32_t)(32 * nb * TL::kPitch);
 
             // S^T of both heads for 32 kv rows (lane owns one q row, 16 of the kv rows)
             f32x16 sa, sb;
-            rowfrag_gemm_dual<D, kPairPipeK>(lds_addr(Ks) + rbase + roff, qa, qb, sa, sb, pace_k);
+            rowfrag_gemm_dual<D, kPairPipeK>(lds_addr(Ks) + rbase + roff, qa, qb, sa, sb, a_hook);
             MA_TICK(3);
 
             // mask (shared by the two heads) and row maxima on the unscaled scores
@@ -275,7 +327,7 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
             if (mode == 1) {  // maxima only
                 ma_ = fmaxf(ma_, mxa);
                 mb_ = fmaxf(mb_, mxb);
-                continue;
+                return;
             }
             if (mode == 0) {
                 // the first visible block sets the reference; a later block that outgrows it by more
@@ -302,12 +354,16 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
 
             // O^T += V^T P^T for both heads: every transposed V fragment feeds two MFMAs
             MA_TICK(4);
-            trfrag_gemm_dual<D, 2, kPairPipeV>(lds_addr(Vs) + tbase + roff, pa, pb, oa, ob, pace_v);
+            trfrag_gemm_dual<D, 2, kPairPipeV>(lds_addr(Vs) + tbase + roff, pa, pb, oa, ob, b_hook);
             MA_TICK(5);
-        }
+        };
+        block(std::integral_constant<int, 0>{});
+        block(std::integral_constant<int, 1>{});
         MA_TICK(6);
+        have = have_next;
     }
 
+    wait_vmem();      // (the chains of the last step have fetched its own tiles once more: no test in the hooks)
     __syncthreads();  // every wave is done with the K/V buffers, and with the flag
     const int redo = *outgrown;
     if (mode == 0 && redo) { mode = 1; continue; }
