@@ -305,7 +305,6 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
     using SQ = DirectStager<D, BM, NW>;
     constexpr int kPaced = (SQ::NL - 1) / NW;
     static_assert(SQ::NL == NW * kPaced + 1 && (2 * KK) % kPaced == 0, "tile runs per wave");
-    constexpr int kEvery = (2 * KK) / kPaced;
     SQ sq;
     sq.init(w, lane);
     uint32_t rc_last;  // the left-over run, whichever wave moves it

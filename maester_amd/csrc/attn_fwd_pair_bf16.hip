@@ -69,6 +69,99 @@ constexpr int kPairPlan[2][2][3] = {{{0, 0, 8}, {1, 0, 4}}, {{1, 4, 4}, {0, 0, 0
 constexpr int kPairPlan[2][2][3] = {{{0, 0, 8}, {0, 0, 0}}, {{0, 0, 0}, {1, 0, 8}}};
 #endif
 
+// The kv steps of one work item, resolved ahead of the loop that runs them.  A wave that has its SIMD to
+// itself pays four cycles for every instruction it issues between two MFMA chains, so whatever a step
+// needs is worked out 64 steps at a time, one candidate step per lane, and kept as a record of
+// ready-made addresses in the wave's own slice of LDS; taking a step is then two broadcast LDS reads
+// and a few v_readfirstlane.
+//   word 0       first kv row | act1 << 29 | act0 << 30 | partial << 31
+//                (act0 / act1: this wave has something to do in the first / second 32-row block)
+//   words 2,3    address of the step's first K row        words 4,5    of its first V row
+//   words 6,7    of the document id of its first row (HAS_DOC)
+// Every wave of a workgroup derives the same sequence of steps (same inputs); only the two block bits
+// are its own.  Nothing a refill needs is kept between refills except the position in the walk: it is
+// derived again from the argument block, so that the step loop holds no registers for it.
+constexpr int kPairRecWords = 8;
+constexpr int kPairRecBytes = 64 * kPairRecWords * 4;  // LDS per wave
+template <bool HAS_DOC>
+struct PairSteps {
+    MA_LDS uint32_t* tab;
+    int cbase, cnt, pos;
+    __device__ __forceinline__ void start(MA_LDS uint32_t* table) { tab = table; cbase = 0; cnt = 0; pos = -1; }
+
+    // the next candidates that hold a step at all; false when the walk is over
+    __device__ __forceinline__ bool refill(const int i, const int hk, const int b, const int w) {
+        KernArgs& a = fresh_args();
+        const int lane = __lane_id();
+        const size_t mrow = (size_t)b * a.T + i;
+        const bool use_rng = HAS_DOC && a.map.block_doc_range != nullptr;
+        const int64_t* rng = use_rng ? a.map.block_doc_range + (size_t)b * (2 * ((a.S + 63) / 64)) * 2 : nullptr;
+        const int qw_lo = i * kTile + 32 * w, qw_hi = qw_lo + 31;
+        DocRange own;  // id range of the wave's own q rows: in the same round trip as the list lengths
+        int np, nf;
+        if (use_rng) scalar_load2_range(a.map.kv_num_blocks + mrow, a.map.full_kv_num_blocks + mrow,
+                                        rng + (size_t)(min(qw_lo, a.S - 1) / MA_DOC_BLOCK) * 2, np, nf, own);
+        else scalar_load2(a.map.kv_num_blocks + mrow, a.map.full_kv_num_blocks + mrow, np, nf);
+        const int n = np + nf, total = n * (kTile / kPairBN);
+        const bool bounded = a.causal || a.window >= 0, windowed = a.window >= 0;
+        const int wlim = windowed ? (int)min(a.window, (int64_t)0x3fffffff) : 0x7fffffff;
+        int vis_lo, vis_hi, blk_lo, blk_hi;
+        visibility_limits(false, i * kTile, i * kTile + kTile - 1, kPairBN, bounded, wlim, windowed, vis_lo, vis_hi);
+        visibility_limits(false, qw_lo, qw_hi, 32, bounded, wlim, windowed, blk_lo, blk_hi);
+        int64_t own_lo = 0, own_hi = 0;
+        if (use_rng) {
+            own_lo = own.lo();
+            own_hi = own.hi();
+        }
+        const int32_t* pl = a.map.kv_indices + mrow * a.T;
+        const int32_t* fl = a.map.full_kv_indices + mrow * a.T;
+        const char* kp = (const char*)((const __bf16*)a.k.ptr + b * a.k.stride_b + hk * a.k.stride_h);
+        const char* vp = (const char*)((const __bf16*)a.v.ptr + b * a.v.stride_b + hk * a.v.stride_h);
+        const uint32_t ksb = (uint32_t)(a.k.stride_s * 2), vsb = (uint32_t)(a.v.stride_s * 2);
+        cnt = 0;
+        while (cnt == 0 && cbase < total) {
+            const int c = cbase + lane;
+            const bool valid = c < total;
+            const int cc = valid ? c : 0;
+            const int idx = cc / (kTile / kPairBN), half = cc - idx * (kTile / kPairBN);
+            const bool partial = idx < np;
+            int tile = 0;
+            if (valid) tile = partial ? pl[idx] : fl[idx - np];
+            const int r0 = tile * kTile + half * kPairBN;
+            const bool vis = valid & (r0 < a.S) & (!partial | ((r0 >= vis_lo) & (r0 <= vis_hi)));
+            bool act0 = (r0 < a.S) & (!partial | ((r0 >= blk_lo) & (r0 <= blk_hi)));
+            bool act1 = (r0 + 32 < a.S) & (!partial | ((r0 + 32 >= blk_lo) & (r0 + 32 <= blk_hi)));
+            if (use_rng && partial && vis) {  // no row of the block shares a document with the wave's own rows
+                const int64_t* e = rng + (size_t)(r0 / 32) * 2;
+                act0 &= (e[0] <= own_hi) & (e[1] >= own_lo);
+                act1 &= (e[2] <= own_hi) & (e[3] >= own_lo);
+            }
+            const uint64_t mask = __ballot(vis);
+            const int at = __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0));
+            if (vis) {
+                const uint64_t ka = (uint64_t)(kp + (uint64_t)(uint32_t)r0 * ksb), va = (uint64_t)(vp + (uint64_t)(uint32_t)r0 * vsb);
+                const uint64_t da = HAS_DOC ? (uint64_t)(a.doc + (size_t)b * a.S + r0) : 0;
+                MA_LDS uint32_t* rec = tab + at * kPairRecWords;
+                *(MA_LDS u32x4*)rec = u32x4{(uint32_t)r0 | ((uint32_t)act1 << 29) | ((uint32_t)act0 << 30) | ((uint32_t)partial << 31), 0u,
+                                            (uint32_t)ka, (uint32_t)(ka >> 32)};
+                *(MA_LDS u32x4*)(rec + 4) = u32x4{(uint32_t)va, (uint32_t)(va >> 32), (uint32_t)da, (uint32_t)(da >> 32)};
+            }
+            cbase += 64;
+            cnt = __builtin_popcountll(mask);
+        }
+        pos = 0;
+        return cnt != 0;
+    }
+    // moves on to the next step: false when the walk is over
+    __device__ __forceinline__ bool advance(const int i, const int hk, const int b, const int w) {
+        if (++pos < cnt) return true;
+        return refill(i, hk, b, w);
+    }
+};
+__device__ __forceinline__ uint64_t pair_uniform64(uint32_t lo, uint32_t hi) {
+    return (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane(lo) | ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane(hi) << 32);
+}
+
 template <int D, bool HAS_DOC>
 __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int wg_id
 #ifdef MA_TICKS
@@ -94,14 +187,12 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
     if (!map_work(wg_id, a.B * a.T, a.T, a.Hkv, GP, a.map.q_tile_order, i, hp, b)) return;
     const int hk = hp / GP;
     const int h0 = hk * G + 2 * (hp % GP);   // the pair is (h0, h0 + 1)
-    const int qw_lo = i * kTile + 32 * w, qw_hi = qw_lo + 31;
+    const int qw_lo = i * kTile + 32 * w;
     const int q = qw_lo + r;
     const bool qvalid = q < a.S;
     const bool bounded = a.causal || a.window >= 0;
 
     const __bf16* qp = (const __bf16*)a.q.ptr + b * a.q.stride_b + h0 * a.q.stride_h;
-    const char* kp = (const char*)((const __bf16*)a.k.ptr + b * a.k.stride_b + hk * a.k.stride_h);
-    const char* vp = (const char*)((const __bf16*)a.v.ptr + b * a.v.stride_b + hk * a.v.stride_h);
     const uint32_t ksb = (uint32_t)(a.k.stride_s * 2), vsb = (uint32_t)(a.v.stride_s * 2);
     const int64_t* drow = HAS_DOC ? a.doc + (size_t)b * a.S : nullptr;
     const int rbase = TL::row_base(lane), tbase = TL::tr_base(lane);
@@ -111,14 +202,6 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
     const bool windowed = a.window >= 0;
     const int wlim = windowed ? (int)min(a.window, (int64_t)0x3fffffff) : 0x7fffffff;
     const float sl2 = a.scale * kLog2e;
-
-    const size_t mrow = (size_t)b * a.T + i;
-    StepTable<BN> st;
-    int blk_lo, blk_hi;
-    visibility_limits(false, qw_lo, qw_hi, 32, bounded, wlim, windowed, blk_lo, blk_hi);
-    const bool use_rng = HAS_DOC && a.map.block_doc_range != nullptr;
-    const int64_t* rng_row = use_rng ? a.map.block_doc_range + (size_t)b * (2 * ((a.S + 63) / 64)) * 2 : nullptr;
-    DocRange own;
 
     // The K and V tiles have the same shape: one set of slots.  Every wave moves the same number of runs
     // of a tile from inside its MFMA chains (kPaced); the run that is left over (a tile is 4 * kPaced + 1
@@ -140,39 +223,40 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
     // straight from global memory into MFMA operand fragments (lane (r, hh): elements 16*kk + 8*hh
     // .. +7 of row qw_lo + r, one 16-byte load each; nothing passes through LDS), then, once the
     // index loads are back, the first K/V tiles -- all in flight together.
+    // (the fields of the current step's word are carried as variables of their own: decoded from the word
+    // inside the loop, the compiler splits the accumulators' live ranges around the skipped-block path
+    // and spills them)
     bool have;
-    int k0;
-    bool partial, act0, act1;  // of the step the walk stands on: tile kind, blocks this wave has work in
-    const char *ksrc = kp, *vsrc = vp;  // its K and V rows
-    MA_LDS uint32_t* steps_slot = (MA_LDS uint32_t*)(lds0 + 4 * TL::bytes(BN) + 2 * BN * 8 + 16) + w * 64;
-    auto walk_init = [&]() {
-        int lo, hi;
-        visibility_limits(false, i * kTile, i * kTile + kTile - 1, BN, bounded, wlim, windowed, lo, hi);
-        int n_partial, n_full;
-        // (the id range of the wave's own rows comes in the same round trip as the list lengths)
-        if (use_rng) scalar_load2_range(a.map.kv_num_blocks + mrow, a.map.full_kv_num_blocks + mrow,
-                                        rng_row + (size_t)(min(qw_lo, a.S - 1) / MA_DOC_BLOCK) * 2, n_partial, n_full, own);
-        else scalar_load2(a.map.kv_num_blocks + mrow, a.map.full_kv_num_blocks + mrow, n_partial, n_full);
-        st.init(a.map.kv_indices + mrow * a.T, n_partial, a.map.full_kv_indices + mrow * a.T, n_full, 1, false, a.S, lo, hi,
-                blk_lo, blk_hi, use_rng ? rng_row : nullptr, use_rng ? own.lo() : 0, use_rng ? own.hi() : 0, steps_slot);
-        st.prime();
+    int k0 = 0;
+    bool partial = false, act0 = false, act1 = false;  // of the step the walk stands on: tile kind, blocks this wave has work in
+    uint64_t k_at = 0, v_at = 0;                       // its K and V rows
+    auto decode = [&](uint32_t word) {
+        k0 = (int)(word & 0xffffffu);
+        partial = (word >> 31) != 0;
+        act0 = (word >> 30) & 1u;
+        act1 = (word >> 29) & 1u;
+    };
+    PairSteps<HAS_DOC> st;
+    // document ids of a partial step's kv rows: every wave loads them for the step after the current
+    // one (no branch: a conditional load would be waited for on the spot), wave 3 writes them to LDS
+    auto load_ids = [&](uint64_t doc_at, int r0) {
+        if (HAS_DOC) kd_next = ((const MA_GLB int64_t*)doc_at)[min(lane, a.S - 1 - r0)];
     };
     auto walk_first = [&]() {
-        have = st.next();
-        k0 = st.r0;
-        partial = st.partial;
-        act0 = st.act0;
-        act1 = st.act1;
+        st.start((MA_LDS uint32_t*)(lds0 + 4 * TL::bytes(BN) + 2 * BN * 8 + 16) + w * (kPairRecBytes / 4));
+        have = st.advance(i, hk, b, w);
         if (have) {
+            MA_LDS uint32_t* rec = st.tab + st.pos * kPairRecWords;
+            const u32x4 x0 = *(MA_LDS u32x4*)rec, x1 = *(MA_LDS u32x4*)(rec + 4);
+            decode(__builtin_amdgcn_readfirstlane(x0[0]));
+            k_at = pair_uniform64(x0[2], x0[3]);
+            v_at = pair_uniform64(x1[0], x1[1]);
             const int rows_valid = min(BN, a.S - k0);
-            ksrc = kp + (uint64_t)(uint32_t)k0 * ksb;
-            vsrc = vp + (uint64_t)(uint32_t)k0 * vsb;
-            sk.issue((const __bf16*)ksrc, Kbuf(0), w, lane, rows_valid, a.k.stride_s);
-            sk.issue((const __bf16*)vsrc, Vbuf(0), w, lane, rows_valid, a.v.stride_s);
-            if (HAS_DOC && partial && tid < BN) kd_next = drow[min(k0 + tid, a.S - 1)];
+            sk.issue((const __bf16*)k_at, Kbuf(0), w, lane, rows_valid, a.k.stride_s);
+            sk.issue((const __bf16*)v_at, Vbuf(0), w, lane, rows_valid, a.v.stride_s);
+            load_ids(pair_uniform64(x1[2], x1[3]), k0);
         }
     };
-    walk_init();
     bf16x8 qa[KK], qb[KK];
     {
         const __bf16* qrow = qp + (int64_t)qc * a.q.stride_s + 8 * hh;
@@ -200,17 +284,21 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
     pin_tiles<0, DB, true>(ob);
     la = lb = 0.f;
     if (mode != 2) ma_ = mb_ = -INFINITY;
-    if (mode) {  // a later pass starts the walk again
-        walk_init();
-        walk_first();
-    }
+    if (mode) walk_first();  // a later pass starts the walk again
 
     for (int n = 0; have; ++n) {
         MA_TICK(0);
         const int cur = n & 1;
         const lds_ptr Ks = Kbuf(cur), Vs = Vbuf(cur);
         MA_LDS int64_t* kdoc = Dbuf(cur);
-        if (HAS_DOC && partial && tid < BN) kdoc[tid] = kd_next;
+        if (HAS_DOC && w == 3) kdoc[lane] = kd_next;
+        const bool have_next = st.advance(i, hk, b, w);
+        u32x4 x0 = {0, 0, 0, 0}, x1 = x0;
+        if (have_next) {  // the record of the next step: read now, picked up behind the barrier
+            MA_LDS uint32_t* rec = st.tab + st.pos * kPairRecWords;
+            x0 = *(MA_LDS u32x4*)rec;
+            x1 = *(MA_LDS u32x4*)(rec + 4);
+        }
         wait_vmem();
         __syncthreads();
         MA_TICK(1);
@@ -218,23 +306,21 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
         const int ck0 = k0;
         const bool cpartial = partial;
         const bool act[2] = {act0, act1};
-        const bool have_next = st.next();
+        uint32_t nword = 0;
         // The tile loads of the next step ride in this step's chains, one run every few MFMAs (see
         // kPairPlan): issued in one burst they fill the memory pipeline and stall the wave with the
         // matrix cores idle.  On the last step of a walk the chains fetch the current tiles once more,
         // into the free half of the ring: cheaper than a test in every hook.
         int nlast = min(BN, a.S - ck0) - 1;
         if (have_next) {
-            k0 = st.r0;
-            partial = st.partial;
-            act0 = st.act0;
-            act1 = st.act1;
-            ksrc = kp + (uint64_t)(uint32_t)k0 * ksb;
-            vsrc = vp + (uint64_t)(uint32_t)k0 * vsb;
-            if (HAS_DOC && partial && tid < BN) kd_next = drow[min(k0 + tid, a.S - 1)];
-            nlast = min(BN, a.S - k0) - 1;
-            if (w == 0) global_to_lds_run_rc(ksrc, rc_last, ksb, nlast, lds_addr(Kbuf(cur ^ 1)) + (SK::NL - 1) * 1024);
-            if (w == 1 && mode != 1) global_to_lds_run_rc(vsrc, rc_last, vsb, nlast, lds_addr(Vbuf(cur ^ 1)) + (SK::NL - 1) * 1024);
+            nword = __builtin_amdgcn_readfirstlane(x0[0]);
+            k_at = pair_uniform64(x0[2], x0[3]);
+            v_at = pair_uniform64(x1[0], x1[1]);
+            const int nk0 = (int)(nword & 0xffffffu);
+            load_ids(pair_uniform64(x1[2], x1[3]), nk0);
+            nlast = min(BN, a.S - nk0) - 1;
+            if (w == 0) global_to_lds_run_rc((const void*)k_at, rc_last, ksb, nlast, lds_addr(Kbuf(cur ^ 1)) + (SK::NL - 1) * 1024);
+            if (w == 1 && mode != 1) global_to_lds_run_rc((const void*)v_at, rc_last, vsb, nlast, lds_addr(Vbuf(cur ^ 1)) + (SK::NL - 1) * 1024);
         }
         const uint32_t kdst = lds_addr(Kbuf(cur ^ 1)), vdst = lds_addr(Vbuf(cur ^ 1));
 
@@ -256,9 +342,9 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
             auto move_run = [&](auto tile_c, auto run_c) {
                 constexpr int run = decltype(run_c)::value;
                 if constexpr (decltype(tile_c)::value == 0)
-                    global_to_lds_run_rc(ksrc, sk.rc[run], ksb, nlast, kdst + w * 1024 + run * (NW * 1024));
+                    global_to_lds_run_rc((const void*)k_at, sk.rc[run], ksb, nlast, kdst + w * 1024 + run * (NW * 1024));
                 else
-                    global_to_lds_run_rc(vsrc, sk.rc[run], vsb, nlast, vdst + w * 1024 + run * (NW * 1024));
+                    global_to_lds_run_rc((const void*)v_at, sk.rc[run], vsb, nlast, vdst + w * 1024 + run * (NW * 1024));
             };
             auto burst_plan = [&](auto plan_c) {
                 constexpr int which = decltype(plan_c)::value;
@@ -360,6 +446,7 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
         block(std::integral_constant<int, 0>{});
         block(std::integral_constant<int, 1>{});
         MA_TICK(6);
+        if (have_next) decode(nword);
         have = have_next;
     }
 
@@ -441,7 +528,7 @@ __global__ __launch_bounds__(kPairThreads) void attn_fwd_pair_bf16_kernel(AttnAr
 
 template <int D, bool HAS_DOC>
 static int pair_dd(const AttnArgs& a, hipStream_t st) {
-    const size_t lds = (size_t)4 * Tile<D>::bytes(kPairBN) + 2 * kPairBN * 8 + 16 + (kPairThreads / 64) * 256;  // K/V ring, kv ids, redo flag + work-queue box, step tables
+    const size_t lds = (size_t)4 * Tile<D>::bytes(kPairBN) + 2 * kPairBN * 8 + 16 + (kPairThreads / 64) * kPairRecBytes;  // K/V ring, kv ids, redo flag + work-queue box, step records
     if (lds > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_pair_bf16_kernel<D, HAS_DOC>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
