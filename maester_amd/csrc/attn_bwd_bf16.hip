@@ -128,6 +128,9 @@ __global__ __launch_bounds__(256) void attn_delta_bf16_kernel(AttnArgs a) {
 #ifndef MA_DKV_PLACE
 #define MA_DKV_PLACE 0
 #endif
+#ifndef MA_DKV_EXP_HOOKS
+#define MA_DKV_EXP_HOOKS 1
+#endif
 #if MA_DKV_PLACE == 0
 constexpr int kDkvPlan[2][2][3] = {{{0, 0, 8}, {0, 0, 0}}, {{1, 0, 8}, {0, 0, 0}}};
 #elif MA_DKV_PLACE == 1
@@ -465,7 +468,24 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
                 }
             }
             const uint32_t roff = (uint32_t)(32 * mb * TL::kPitch);
+#if MA_DKV_EXP_HOOKS
+            // The two products run one after the other so that the exponentials of S (a quarter-rate
+            // instruction each) are taken in the shadow of the dP MFMAs: one value per MFMA, from the
+            // second MFMA after S is complete; what does not fit follows the chain.
+            constexpr int kFirstExp = KK + 2, kHooked = (2 * KK - kFirstExp) < 16 ? (2 * KK - kFirstExp) : 16;
+            auto chain_hook = [&](auto idx) {
+                constexpr int i = decltype(idx)::value;
+                a_hook(idx);
+                if constexpr (i >= kFirstExp && i - kFirstExp < 16) s[i - kFirstExp] = fast_exp2(s[i - kFirstExp] * sl2);
+            };
+            rowfrag_gemm2<D, kBPipe, false, false, decltype(chain_hook)&, true, true>(lds_addr(Qs) + rbase + roff, kf, s, lds_addr(Gs) + rbase + roff, vf, dp, chain_hook);
+#pragma unroll
+            for (int v = kHooked; v < 16; ++v) s[v] = fast_exp2(s[v] * sl2);
+#else
             rowfrag_gemm2<D, kBPipe, false, false, decltype(a_hook)&, false, true>(lds_addr(Qs) + rbase + roff, kf, s, lds_addr(Gs) + rbase + roff, vf, dp, a_hook);
+#pragma unroll
+            for (int v = 0; v < 16; ++v) s[v] = fast_exp2(s[v] * sl2);
+#endif
             MA_TICK(3);
 
             bf16x8 pf[2], dsf[2];
@@ -492,7 +512,7 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         const int v = 4 * g4 + e;
-                        float p = fast_exp2(s[v] * sl2);
+                        float p = s[v];  // exp2((S - lse / scale) * scale * log2 e) by now
                         if (MASKED) {
                             bool ok = (t0 + (unsigned)(8 * g4 + e) <= span) & some;
                             if (HAS_DOC) ok = ok & (ids[e] == dock);
