@@ -652,16 +652,15 @@ __device__ __forceinline__ void attn_bwd_dq_bf16_item(KernArgs& a, const int wg_
     const bool use_rng = HAS_DOC && a.map.block_doc_range != nullptr;
     const int64_t* rng_row = use_rng ? a.map.block_doc_range + (size_t)b * (2 * ((a.S + 63) / 64)) * 2 : nullptr;
     DocRange own;
-    if (use_rng) {  // (load and wait stay adjacent: the registers of a scalar load in flight must not be touched)
-        own.load(rng_row + (size_t)(min(qw_lo, a.S - 1) / MA_DOC_BLOCK) * 2);
-        own.ready();
-    }
     StepTable<BN> st;
     {
         int lo, hi;
         visibility_limits(false, i * kTile, i * kTile + kTile - 1, BN, bounded, wlim, windowed, lo, hi);
         int n_partial, n_full;
-        scalar_load2(a.map.kv_num_blocks + mrow, a.map.full_kv_num_blocks + mrow, n_partial, n_full);
+        // (the id range of the wave's own rows comes in the same round trip as the list lengths)
+        if (use_rng) scalar_load2_range(a.map.kv_num_blocks + mrow, a.map.full_kv_num_blocks + mrow,
+                                        rng_row + (size_t)(min(qw_lo, a.S - 1) / MA_DOC_BLOCK) * 2, n_partial, n_full, own);
+        else scalar_load2(a.map.kv_num_blocks + mrow, a.map.full_kv_num_blocks + mrow, n_partial, n_full);
         st.init(a.map.kv_indices + mrow * a.T, n_partial, a.map.full_kv_indices + mrow * a.T, n_full, 1, false, a.S, lo, hi,
                 blk_lo, blk_hi, rng_row, use_rng ? own.lo() : 0, use_rng ? own.hi() : 0,
                 (MA_LDS uint32_t*)(lds0 + 4 * TL::bytes(BN) + 2 * BN * 8 + 16) + w * 64);
@@ -892,17 +891,16 @@ __device__ __forceinline__ void attn_bwd_dq_ds_bf16_item(KernArgs& a, const int 
     const bool use_rng = HAS_DOC && a.map.block_doc_range != nullptr;
     const int64_t* rng_row = use_rng ? a.map.block_doc_range + (size_t)b * (2 * ((a.S + 63) / 64)) * 2 : nullptr;
     DocRange own;
-    if (use_rng) {  // (load and wait stay adjacent: the registers of a scalar load in flight must not be touched)
-        own.load(rng_row + (size_t)(min(qw_lo, a.S - 1) / MA_DOC_BLOCK) * 2);
-        own.ready();
-    }
     StepTable<BN, true> st;
     st.numbering(a.map.tile_slot, ((int64_t)b * a.T + i) * a.T, 1);     // tile (i, j) of this batch row, j walked
     {
         int lo, hi;
         visibility_limits(false, i * kTile, i * kTile + kTile - 1, BN, bounded, wlim, windowed, lo, hi);
         int n_partial, n_full;
-        scalar_load2(a.map.kv_num_blocks + mrow, a.map.full_kv_num_blocks + mrow, n_partial, n_full);
+        // (the id range of the wave's own rows comes in the same round trip as the list lengths)
+        if (use_rng) scalar_load2_range(a.map.kv_num_blocks + mrow, a.map.full_kv_num_blocks + mrow,
+                                        rng_row + (size_t)(min(qw_lo, a.S - 1) / MA_DOC_BLOCK) * 2, n_partial, n_full, own);
+        else scalar_load2(a.map.kv_num_blocks + mrow, a.map.full_kv_num_blocks + mrow, n_partial, n_full);
         st.init(a.map.kv_indices + mrow * a.T, n_partial, a.map.full_kv_indices + mrow * a.T, n_full, 1, false, a.S, lo, hi,
                 blk_lo, blk_hi, rng_row, use_rng ? own.lo() : 0, use_rng ? own.hi() : 0,
                 (MA_LDS uint32_t*)(lds0 + 2 * TL::bytes(BN) + 2 * TS::bytes(BN) + 16) + w * 128);
@@ -1004,17 +1002,16 @@ __device__ __forceinline__ void attn_bwd_dq_ds_pair_bf16_item(KernArgs& a, const
     const bool use_rng = HAS_DOC && a.map.block_doc_range != nullptr;
     const int64_t* rng_row = use_rng ? a.map.block_doc_range + (size_t)b * (2 * ((a.S + 63) / 64)) * 2 : nullptr;
     DocRange own;
-    if (use_rng) {  // (load and wait stay adjacent: the registers of a scalar load in flight must not be touched)
-        own.load(rng_row + (size_t)(min(qw_lo, a.S - 1) / MA_DOC_BLOCK) * 2);
-        own.ready();
-    }
     StepTable<BN, true> st;
     st.numbering(a.map.tile_slot, ((int64_t)b * a.T + i) * a.T, 1);     // tile (i, j) of this batch row, j walked
     {
         int lo, hi;
         visibility_limits(false, i * kTile, i * kTile + kTile - 1, BN, bounded, wlim, windowed, lo, hi);
         int n_partial, n_full;
-        scalar_load2(a.map.kv_num_blocks + mrow, a.map.full_kv_num_blocks + mrow, n_partial, n_full);
+        // (the id range of the wave's own rows comes in the same round trip as the list lengths)
+        if (use_rng) scalar_load2_range(a.map.kv_num_blocks + mrow, a.map.full_kv_num_blocks + mrow,
+                                        rng_row + (size_t)(min(qw_lo, a.S - 1) / MA_DOC_BLOCK) * 2, n_partial, n_full, own);
+        else scalar_load2(a.map.kv_num_blocks + mrow, a.map.full_kv_num_blocks + mrow, n_partial, n_full);
         st.init(a.map.kv_indices + mrow * a.T, n_partial, a.map.full_kv_indices + mrow * a.T, n_full, 1, false, a.S, lo, hi,
                 blk_lo, blk_hi, rng_row, use_rng ? own.lo() : 0, use_rng ? own.hi() : 0,
                 (MA_LDS uint32_t*)(lds0 + 2 * kStage + 16) + w * 128);
