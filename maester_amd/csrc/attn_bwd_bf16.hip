@@ -274,23 +274,18 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
     const int64_t dock = HAS_DOC ? drow[kvc] : 0;
     const int wlim = a.window >= 0 ? (int)min(a.window, (int64_t)0x3fffffff) : 0x7fffffff;
 
-    // K and V rows of the workgroup come in through LDS (coalesced) and stay in registers
+    // K and V rows of the wave go straight from global memory into MFMA operand fragments (lane (r, hh):
+    // elements 16*kk + 8*hh .. +7 of row kw_lo + r, one 16-byte load each; rows past the end of the
+    // sequence re-read the last valid row and are masked).  Nothing waits for them here: the walk is
+    // resolved and the first tiles are requested while they are on their way.
     bf16x8 kf[KK], vf[KK];
     {
-        DirectStager<D, kTile, NW> sk, sv;
-        sk.init(w, lane);
-        sv.init(w, lane);
-        const int rows_valid = min(kTile, S - j * kTile);
-        sk.issue(kp + (int64_t)j * kTile * a.k.stride_s, Qbuf(0), w, lane, rows_valid, a.k.stride_s);
-        sv.issue(vp + (int64_t)j * kTile * a.v.stride_s, Qbuf(1), w, lane, rows_valid, a.v.stride_s);
-        wait_vmem();
-        __syncthreads();
+        const __bf16* krow = kp + (int64_t)kvc * a.k.stride_s + 8 * hh;
+        const __bf16* vrow = vp + (int64_t)kvc * a.v.stride_s + 8 * hh;
 #pragma unroll
-        for (int kk = 0; kk < KK; ++kk) {
-            kf[kk] = TL::row_frag(Qbuf(0), rbase, 32 * w, kk);
-            vf[kk] = TL::row_frag(Qbuf(1), rbase, 32 * w, kk);
-        }
-        __syncthreads();
+        for (int kk = 0; kk < KK; ++kk) kf[kk] = *(const bf16x8*)(krow + 16 * kk);
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) vf[kk] = *(const bf16x8*)(vrow + 16 * kk);
     }
 
     f32x16 dkacc[DB], dvacc[DB];
