@@ -467,8 +467,10 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
         lds_ptr Os = lds0 + w * 32 * kPitchO;
         constexpr int CH = D / 8, RPI = 64 / CH;
         const int rsub = lane / CH, c = lane % CH;
-#pragma unroll 1
-        for (int hsel = 0; hsel < 2; ++hsel) {
+        // (one copy of the code per head: picked at run time, every element would be read from both
+        // accumulators and selected)
+        static_for<0, 2>([&](auto hsel_c) {
+            constexpr int hsel = decltype(hsel_c)::value;
             const float l = hsel ? lb : la, m = hsel ? mb_ : ma_;
             const float inv = l > 0.f ? 1.0f / l : 0.f;
 #pragma unroll
@@ -490,7 +492,7 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
             }
             if (qvalid && hh == 0)
                 a.lse[((size_t)b * a.Hq + h0 + hsel) * a.S + q] = l > 0.f ? (m + __log2f(l)) * kLn2 : -INFINITY;
-        }
+        });
     }
 }
 
