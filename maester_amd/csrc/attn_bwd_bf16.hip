@@ -26,7 +26,8 @@
 namespace ma {
 
 #ifdef MA_TICKS
-// debug build only: cycles a wave spends between two marked points of the dK/dV kernel
+// measurement builds only (maester_amd/kernel_ticks.py): cycles a wave spends between two of the marks
+// MA_TICK(n) of the dK/dV kernel; in the library the marks compile to nothing
 __device__ unsigned long long ma_dbg_ticks[4];
 struct Ticks {
     unsigned long long begin = 0, acc = 0;

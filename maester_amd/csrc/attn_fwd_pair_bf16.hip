@@ -26,7 +26,8 @@
 namespace ma {
 
 #ifdef MA_TICKS
-// debug build only: cycles a wave spends between two marked points of the kernel
+// measurement builds only (maester_amd/kernel_ticks.py): cycles a wave spends between two of the marks
+// MA_TICK(n) of the kernel; in the library the marks compile to nothing
 __device__ unsigned long long ma_dbg_ticks_fwd[4];
 struct TicksF {
     unsigned long long begin = 0, acc = 0;
@@ -379,8 +380,7 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
             rowfrag_gemm_dual<D, kPairPipeK>(lds_addr(Ks) + rbase + roff, qa, qb, sa, sb, a_hook);
             MA_TICK(3);
 
-            // mask (shared by the two heads) and row maxima on the unscaled scores
-            float mxa = -INFINITY, mxb = -INFINITY;
+            // mask (shared by the two heads)
             if (cpartial) {
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
@@ -397,31 +397,35 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
                         if (HAS_DOC) ok = ok & (ids[e] == docq);
                         sa[v] = ok ? sa[v] : -INFINITY;
                         sb[v] = ok ? sb[v] : -INFINITY;
-                        mxa = fmaxf(mxa, sa[v]);
-                        mxb = fmaxf(mxb, sb[v]);
                     }
                 }
-            } else {
+            }
+            // Once every row of the wave has its reference, a block needs no row maxima: the scores
+            // are exponentiated against the references and a row that outgrows the slack shows in its
+            // sum (a sum above 2^kSlack sends the workgroup into the redo, as a single term would).
+            const bool settled = (mode != 1) & !__any((ma_ == -INFINITY) | (mb_ == -INFINITY));
+            if (!settled) {
+                float mxa = -INFINITY, mxb = -INFINITY;  // row maxima on the unscaled scores
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     mxa = fmaxf(mxa, sa[v]);
                     mxb = fmaxf(mxb, sb[v]);
                 }
-            }
-            mxa = fmaxf(mxa, xor32(mxa)) * sl2;   // the (positive) scale goes into the exponent's multiply-add
-            mxb = fmaxf(mxb, xor32(mxb)) * sl2;
-            if (mode == 1) {  // maxima only
-                ma_ = fmaxf(ma_, mxa);
-                mb_ = fmaxf(mb_, mxb);
-                return;
-            }
-            if (mode == 0) {
-                // the first visible block sets the reference; a later block that outgrows it by more
-                // than kSlack log2 units sends the workgroup into the two-pass redo
-                const bool late = ((ma_ != -INFINITY) & (mxa > ma_ + kSlack)) | ((mb_ != -INFINITY) & (mxb > mb_ + kSlack));
-                if (__any(late) && lane == 0) *outgrown = 1;
-                ma_ = ma_ == -INFINITY ? mxa : ma_;
-                mb_ = mb_ == -INFINITY ? mxb : mb_;
+                mxa = fmaxf(mxa, xor32(mxa)) * sl2;   // the (positive) scale goes into the exponent's multiply-add
+                mxb = fmaxf(mxb, xor32(mxb)) * sl2;
+                if (mode == 1) {  // maxima only
+                    ma_ = fmaxf(ma_, mxa);
+                    mb_ = fmaxf(mb_, mxb);
+                    return;
+                }
+                if (mode == 0) {
+                    // the first visible block sets the reference; a later block that outgrows it by more
+                    // than kSlack log2 units sends the workgroup into the two-pass redo
+                    const bool late = ((ma_ != -INFINITY) & (mxa > ma_ + kSlack)) | ((mb_ != -INFINITY) & (mxb > mb_ + kSlack));
+                    if (__any(late) && lane == 0) *outgrown = 1;
+                    ma_ = ma_ == -INFINITY ? mxa : ma_;
+                    mb_ = mb_ == -INFINITY ? mxb : mb_;
+                }
             }
             const float mua = ma_ == -INFINITY ? 0.f : ma_, mub = mb_ == -INFINITY ? 0.f : mb_;
             float rsa = 0.f, rsb = 0.f;
@@ -435,8 +439,13 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
                 pa[v >> 3][v & 7] = (__bf16)x;
                 pb[v >> 3][v & 7] = (__bf16)y;
             }
-            la += rsa + xor32(rsa);
-            lb += rsb + xor32(rsb);
+            if (settled && mode == 0) {
+                constexpr float kTooLarge = 4294967296.0f;  // 2^kSlack
+                static_assert(kSlack == 32.0f, "threshold of the row sums");
+                if (__any((rsa > kTooLarge) | (rsb > kTooLarge)) && lane == 0) *outgrown = 1;
+            }
+            la += rsa;  // the lane's own 16 kv rows of the block; the two lanes of a q row are added at the end
+            lb += rsb;
 
             // O^T += V^T P^T for both heads: every transposed V fragment feeds two MFMAs
             MA_TICK(4);
@@ -471,7 +480,8 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
         // accumulators and selected)
         static_for<0, 2>([&](auto hsel_c) {
             constexpr int hsel = decltype(hsel_c)::value;
-            const float l = hsel ? lb : la, m = hsel ? mb_ : ma_;
+            const float lp = hsel ? lb : la, m = hsel ? mb_ : ma_;
+            const float l = lp + xor32(lp);
             const float inv = l > 0.f ? 1.0f / l : 0.f;
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
