@@ -281,6 +281,10 @@ __device__ __forceinline__ void rowfrag_gemm2(uint32_t row_addr0, const bf16x8* 
         constexpr int i = decltype(idx)::value;
         step(idx);
         if constexpr (i + P < N) rd(std::integral_constant<int, i + P>{});
+        // SEQ: acc0 is final after MFMA KK-1 and may be read by the vector ALU once two more MFMAs have
+        // been issued.  Pinning it here keeps whatever the hooks do with it below this point (their
+        // arithmetic is ordinary code, which the compiler would otherwise move up to MFMA KK-1).
+        if constexpr (SEQ && i == KK + 1) asm volatile("" : "+v"(acc0));
         hook(idx);
     });
     mfma_fence();
