@@ -74,11 +74,19 @@ __device__ __forceinline__ void store_tile_T(lds_ptr scratch, const f32x16* acc,
     }
     constexpr int CH = D / 8, RPI = 64 / CH;
     const int rsub = lane / CH, c = lane % CH;
+    // all rows leave LDS first, then go out (one LDS round trip; 32-bit offsets from a uniform base)
+    MA_GLB char* g0 = (MA_GLB char*)(gbase + (int64_t)row0 * stride);
+    const uint32_t row_bytes = (uint32_t)(stride * 2);
+    u32x4 val[32 / RPI];
 #pragma unroll
-    for (int it = 0; it < 32 / RPI; ++it) {
-        const int row = it * RPI + rsub;
-        const u32x4 val = *(MA_LDS u32x4*)(scratch + row * kPitchO + c * 16);
-        if (row0 + row < rows_end) *(u32x4*)(gbase + (int64_t)(row0 + row) * stride + c * 8) = val;
+    for (int it = 0; it < 32 / RPI; ++it) val[it] = *(MA_LDS u32x4*)(scratch + (it * RPI + rsub) * kPitchO + c * 16);
+    if (row0 + 31 < rows_end) {
+#pragma unroll
+        for (int it = 0; it < 32 / RPI; ++it) *(MA_GLB u32x4*)(g0 + (uint32_t)(it * RPI + rsub) * row_bytes + c * 16) = val[it];
+    } else {
+#pragma unroll
+        for (int it = 0; it < 32 / RPI; ++it)
+            if (row0 + it * RPI + rsub < rows_end) *(MA_GLB u32x4*)(g0 + (uint32_t)(it * RPI + rsub) * row_bytes + c * 16) = val[it];
     }
 }
 
@@ -149,8 +157,13 @@ struct DkvSteps {
     int cbase, cnt, pos;
     __device__ __forceinline__ void start(MA_LDS uint32_t* table) { tab = table; cbase = 0; cnt = 0; pos = -1; }
 
-    // the next candidates that hold a step at all; false when the walk is over
-    __device__ __forceinline__ bool refill(const int j, const int hk, const int b, const int w) {
+    // the next candidates that hold a step at all; false when the walk is over.
+    // FIRST (an item's first fill): the candidates are scanned at least once, and `mid1` / `mid2` run
+    // while the scan's two dependent loads (list entries, then id ranges and workspace slots) are on
+    // their way -- the item's own operand loads go there, so that the round trips do not queue up behind
+    // them.  Every load of the scan is unconditional (a load under a condition is waited for on the spot).
+    template <bool FIRST, class F1, class F2>
+    __device__ __forceinline__ bool refill(const int j, const int hk, const int b, const int w, F1&& mid1, F2&& mid2) {
         KernArgs& a = fresh_args();
         const int lane = __lane_id();
         const int G = a.Hq / a.Hkv;
@@ -176,25 +189,50 @@ struct DkvSteps {
         }
         const int32_t* pl = a.map.q_indices + mrow * a.T;
         const int32_t* fl = a.map.full_q_indices + mrow * a.T;
+        const void* kbase = (const void*)((const __bf16*)a.k.ptr + b * a.k.stride_b + hk * a.k.stride_h);  // readable, at least a row long
         cnt = 0;
-        while (cnt == 0 && cbase < total) {
+        auto scan = [&](auto first_c) {
+            constexpr bool first = decltype(first_c)::value;
             const int c = cbase + lane;
-            const bool valid = c < total;
+            const bool valid = (c < total) & (n > 0);
             const int cc = valid ? c : 0;
-            const int rep = cc / per_pass, wi = cc - rep * per_pass;
+            const int rep = cc / max(per_pass, 1), wi = cc - rep * per_pass;
             const int it = wi / (kTile / kStep), half = wi - it * (kTile / kStep);
-            const int idx = n - 1 - it;  // from the last q tile down: the workgroups of a document start on the same tiles
+            const int idx = max(n - 1 - it, 0);  // from the last q tile down: the workgroups of a document start on the same tiles
             const bool partial = idx < np;
-            int tile = 0;
-            if (valid) tile = partial ? pl[idx] : fl[idx - np];
+            const int32_t* entry = partial ? pl + idx : fl + (idx - np);  // (no candidate: the first entry of a list, unused)
+            int tile = *(const MA_GLB int32_t*)entry;
+            if constexpr (first) {
+                asm volatile("" ::: "memory");
+                mid1();
+                asm volatile("" ::: "memory");
+            }
+            tile = valid ? tile : 0;
             const int r0 = tile * kTile + half * kStep;
             const bool vis = valid & (r0 < a.S) & (!partial | ((r0 >= vis_lo) & (r0 <= vis_hi)));
             bool act0 = (r0 < a.S) & (!partial | ((r0 >= blk_lo) & (r0 <= blk_hi)));
             bool act1 = (r0 + 32 < a.S) & (!partial | ((r0 + 32 >= blk_lo) & (r0 + 32 <= blk_hi)));
-            if (use_rng && partial && vis) {  // no row of the block shares a document with the wave's own rows
-                const int64_t* e = rng + (size_t)(r0 / 32) * 2;
-                act0 &= (e[0] <= own_hi) & (e[1] >= own_lo);
-                act1 &= (e[2] <= own_hi) & (e[3] >= own_lo);
+            // what depends on the tile's number goes out together: the id ranges of the step's two blocks
+            // and the tile's slot in the dS workspace.  Where there is nothing to look up (no range table,
+            // a full tile, no step) the range load reads the head of the K tensor and its result is not used.
+            uint32_t tslot = 0;
+            if constexpr (WRITE_DS) tslot = (uint32_t)((const MA_GLB int32_t*)a.map.tile_slot)[((int64_t)b * a.T + tile) * a.T + j];
+            i64x2 e0 = {0, 0}, e1 = {0, 0};
+            bool look = false;
+            if constexpr (HAS_DOC) {
+                look = use_rng & partial & vis;
+                const MA_GLB i64x2* e = (const MA_GLB i64x2*)(look ? (const void*)(rng + (size_t)(r0 / 32) * 2) : kbase);
+                e0 = e[0];
+                e1 = e[1];
+            }
+            if constexpr (first) {
+                asm volatile("" ::: "memory");
+                mid2();
+                asm volatile("" ::: "memory");
+            }
+            if constexpr (HAS_DOC) {  // no row of the block shares a document with the wave's own rows
+                act0 &= !look | ((e0[0] <= own_hi) & (e0[1] >= own_lo));
+                act1 &= !look | ((e1[0] <= own_hi) & (e1[1] >= own_lo));
             }
             const uint64_t mask = __ballot(vis);
             const int at = __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0));
@@ -206,7 +244,6 @@ struct DkvSteps {
                 const uint64_t la = (uint64_t)(a.lse + row), ea = (uint64_t)(a.delta + row);
                 uint64_t da = 0;
                 if (WRITE_DS) {
-                    const uint32_t tslot = (uint32_t)a.map.tile_slot[((int64_t)b * a.T + tile) * a.T + j];
                     da = (uint64_t)((char*)a.ds + ((uint64_t)(uint32_t)h * (uint64_t)a.ds_tiles + tslot) * (kTile * kTile * 2) + (r0 & (kTile - 1)) * 2);
                 }
                 MA_LDS uint32_t* rec = tab + at * kDkvRecWords;
@@ -217,14 +254,21 @@ struct DkvSteps {
             }
             cbase += 64;
             cnt = __builtin_popcountll(mask);
-        }
+        };
+        if constexpr (FIRST) scan(std::true_type{});
+        while (cnt == 0 && cbase < total) scan(std::false_type{});
         pos = 0;
         return cnt != 0;
     }
     // moves on to the next step: false when the walk is over
     __device__ __forceinline__ bool advance(const int j, const int hk, const int b, const int w) {
         if (++pos < cnt) return true;
-        return refill(j, hk, b, w);
+        return refill<false>(j, hk, b, w, [] {}, [] {});
+    }
+    // the first step of an item (call after start())
+    template <class F1, class F2>
+    __device__ __forceinline__ bool advance_first(const int j, const int hk, const int b, const int w, F1&& mid1, F2&& mid2) {
+        return refill<true>(j, hk, b, w, mid1, mid2);
     }
 };
 __device__ __forceinline__ uint64_t uniform64(uint32_t lo, uint32_t hi) {
@@ -280,14 +324,16 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
     // sequence re-read the last valid row and are masked).  Nothing waits for them here: the walk is
     // resolved and the first tiles are requested while they are on their way.
     bf16x8 kf[KK], vf[KK];
-    {
-        const __bf16* krow = kp + (int64_t)kvc * a.k.stride_s + 8 * hh;
-        const __bf16* vrow = vp + (int64_t)kvc * a.v.stride_s + 8 * hh;
+    const __bf16* krow = kp + (int64_t)kvc * a.k.stride_s + 8 * hh;
+    const __bf16* vrow = vp + (int64_t)kvc * a.v.stride_s + 8 * hh;
+    auto load_kf = [&]() {
 #pragma unroll
         for (int kk = 0; kk < KK; ++kk) kf[kk] = *(const bf16x8*)(krow + 16 * kk);
+    };
+    auto load_vf = [&]() {
 #pragma unroll
         for (int kk = 0; kk < KK; ++kk) vf[kk] = *(const bf16x8*)(vrow + 16 * kk);
-    }
+    };
 
     f32x16 dkacc[DB], dvacc[DB];
 #pragma unroll
@@ -345,7 +391,7 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
         act0 = (word >> 30) & 1u;
         act1 = (word >> 29) & 1u;
     };
-    bool have = st.advance(j, hk, b, w);
+    bool have = st.advance_first(j, hk, b, w, load_kf, load_vf);
     if (have) {
         MA_LDS uint32_t* rec = st.tab + st.pos * kDkvRecWords;
         const u32x4 x0 = *(MA_LDS u32x4*)rec, x1 = *(MA_LDS u32x4*)(rec + 4), x2 = *(MA_LDS u32x4*)(rec + 8);
@@ -392,7 +438,7 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
         // one run every four MFMAs (Q tile from the S / dP chain, dO tile from the dV / dK chain): issued
         // in one burst they fill the memory pipeline and stall the wave with the matrix cores idle, and
         // issued later in the step they have not landed when the next step begins.
-        int nlast = min(BM, S - cq0) - 1;
+        int nlast = 0;  // (the last step of a walk: its chains fetch the first row of the current tiles again, see below)
         if (have_next) {
             nflags = __builtin_amdgcn_readfirstlane(x0[0]);
             nq_at = uniform64(x0[2], x0[3]);
@@ -549,7 +595,8 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
         have = have_next;
     }
 
-    wait_vmem();      // (the chains of the last step have fetched its own tiles once more: no test in the hooks)
+    wait_vmem();      // (the chains of the last step have fetched the first row of its own tiles over and over, into the
+                      // free half of the ring: no test in the hooks, and nothing that leaves the L1)
     __syncthreads();  // everyone is done with the tiles: reuse the ring as store scratch
     mfma_fence();
     {

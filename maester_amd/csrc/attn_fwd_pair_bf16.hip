@@ -90,8 +90,13 @@ struct PairSteps {
     int cbase, cnt, pos;
     __device__ __forceinline__ void start(MA_LDS uint32_t* table) { tab = table; cbase = 0; cnt = 0; pos = -1; }
 
-    // the next candidates that hold a step at all; false when the walk is over
-    __device__ __forceinline__ bool refill(const int i, const int hk, const int b, const int w) {
+    // the next candidates that hold a step at all; false when the walk is over.
+    // FIRST (an item's first fill): the candidates are scanned at least once, and `mid1` / `mid2` run
+    // while the scan's two dependent loads (list entries, then id ranges of the blocks) are on their way
+    // -- the item's own operand loads go there, so that the round trips do not queue up behind them.
+    // Every load of the scan is unconditional (a load under a condition is waited for on the spot).
+    template <bool FIRST, class F1, class F2>
+    __device__ __forceinline__ bool refill(const int i, const int hk, const int b, const int w, F1&& mid1, F2&& mid2) {
         KernArgs& a = fresh_args();
         const int lane = __lane_id();
         const size_t mrow = (size_t)b * a.T + i;
@@ -120,22 +125,41 @@ struct PairSteps {
         const char* vp = (const char*)((const __bf16*)a.v.ptr + b * a.v.stride_b + hk * a.v.stride_h);
         const uint32_t ksb = (uint32_t)(a.k.stride_s * 2), vsb = (uint32_t)(a.v.stride_s * 2);
         cnt = 0;
-        while (cnt == 0 && cbase < total) {
+        auto scan = [&](auto first_c) {
+            constexpr bool first = decltype(first_c)::value;
             const int c = cbase + lane;
             const bool valid = c < total;
             const int cc = valid ? c : 0;
             const int idx = cc / (kTile / kPairBN), half = cc - idx * (kTile / kPairBN);
             const bool partial = idx < np;
-            int tile = 0;
-            if (valid) tile = partial ? pl[idx] : fl[idx - np];
+            const int32_t* entry = partial ? pl + idx : fl + (idx - np);  // (no candidate: the first entry of a list, unused)
+            int tile = *(const MA_GLB int32_t*)entry;
+            if constexpr (first) {
+                asm volatile("" ::: "memory");
+                mid1();
+                asm volatile("" ::: "memory");
+            }
+            tile = valid ? tile : 0;
             const int r0 = tile * kTile + half * kPairBN;
             const bool vis = valid & (r0 < a.S) & (!partial | ((r0 >= vis_lo) & (r0 <= vis_hi)));
             bool act0 = (r0 < a.S) & (!partial | ((r0 >= blk_lo) & (r0 <= blk_hi)));
             bool act1 = (r0 + 32 < a.S) & (!partial | ((r0 + 32 >= blk_lo) & (r0 + 32 <= blk_hi)));
-            if (use_rng && partial && vis) {  // no row of the block shares a document with the wave's own rows
-                const int64_t* e = rng + (size_t)(r0 / 32) * 2;
-                act0 &= (e[0] <= own_hi) & (e[1] >= own_lo);
-                act1 &= (e[2] <= own_hi) & (e[3] >= own_lo);
+            if constexpr (HAS_DOC) {
+                // id ranges of the step's two blocks; where there is nothing to look up (no range table, a full
+                // tile, no step) the load reads the head of the K tensor instead and its result is not used
+                const bool look = use_rng & partial & vis;
+                const MA_GLB i64x2* e = (const MA_GLB i64x2*)(look ? (const void*)(rng + (size_t)(r0 / 32) * 2) : (const void*)kp);
+                const i64x2 e0 = e[0], e1 = e[1];
+                if constexpr (first) {
+                    asm volatile("" ::: "memory");
+                    mid2();
+                    asm volatile("" ::: "memory");
+                }
+                // no row of the block shares a document with the wave's own rows
+                act0 &= !look | ((e0[0] <= own_hi) & (e0[1] >= own_lo));
+                act1 &= !look | ((e1[0] <= own_hi) & (e1[1] >= own_lo));
+            } else if constexpr (first) {
+                mid2();
             }
             const uint64_t mask = __ballot(vis);
             const int at = __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0));
@@ -149,14 +173,21 @@ struct PairSteps {
             }
             cbase += 64;
             cnt = __builtin_popcountll(mask);
-        }
+        };
+        if constexpr (FIRST) scan(std::true_type{});
+        while (cnt == 0 && cbase < total) scan(std::false_type{});
         pos = 0;
         return cnt != 0;
     }
     // moves on to the next step: false when the walk is over
     __device__ __forceinline__ bool advance(const int i, const int hk, const int b, const int w) {
         if (++pos < cnt) return true;
-        return refill(i, hk, b, w);
+        return refill<false>(i, hk, b, w, [] {}, [] {});
+    }
+    // the first step of an item (call after start())
+    template <class F1, class F2>
+    __device__ __forceinline__ bool advance_first(const int i, const int hk, const int b, const int w, F1&& mid1, F2&& mid2) {
+        return refill<true>(i, hk, b, w, mid1, mid2);
     }
 };
 __device__ __forceinline__ uint64_t pair_uniform64(uint32_t lo, uint32_t hi) {
@@ -186,6 +217,7 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
     const int G = a.Hq / a.Hkv, GP = G / 2;  // head pairs per kv head
     int i, hp, b;
     if (!map_work(wg_id, a.B * a.T, a.T, a.Hkv, GP, a.map.q_tile_order, i, hp, b)) return;
+    MA_TICK(9);
     const int hk = hp / GP;
     const int h0 = hk * G + 2 * (hp % GP);   // the pair is (h0, h0 + 1)
     const int qw_lo = i * kTile + 32 * w;
@@ -243,9 +275,21 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
     auto load_ids = [&](uint64_t doc_at, int r0) {
         if (HAS_DOC) kd_next = ((const MA_GLB int64_t*)doc_at)[min(lane, a.S - 1 - r0)];
     };
-    auto walk_first = [&]() {
+    bf16x8 qa[KK], qb[KK];
+    const __bf16* qrow = qp + (int64_t)qc * a.q.stride_s + 8 * hh;
+    auto load_qa = [&]() {
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) qa[kk] = *(const bf16x8*)(qrow + 16 * kk);
+    };
+    auto load_qb = [&]() {
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) qb[kk] = *(const bf16x8*)(qrow + a.q.stride_h + 16 * kk);
+    };
+    auto walk_first = [&](auto first_c) {
         st.start((MA_LDS uint32_t*)(lds0 + 4 * TL::bytes(BN) + 2 * BN * 8 + 16) + w * (kPairRecBytes / 4));
-        have = st.advance(i, hk, b, w);
+        if constexpr (decltype(first_c)::value) have = st.advance_first(i, hk, b, w, load_qa, load_qb);
+        else have = st.advance(i, hk, b, w);
+        MA_TICK(17);
         if (have) {
             MA_LDS uint32_t* rec = st.tab + st.pos * kPairRecWords;
             const u32x4 x0 = *(MA_LDS u32x4*)rec, x1 = *(MA_LDS u32x4*)(rec + 4);
@@ -258,15 +302,9 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
             load_ids(pair_uniform64(x1[2], x1[3]), k0);
         }
     };
-    bf16x8 qa[KK], qb[KK];
-    {
-        const __bf16* qrow = qp + (int64_t)qc * a.q.stride_s + 8 * hh;
-#pragma unroll
-        for (int kk = 0; kk < KK; ++kk) qa[kk] = *(const bf16x8*)(qrow + 16 * kk);
-#pragma unroll
-        for (int kk = 0; kk < KK; ++kk) qb[kk] = *(const bf16x8*)(qrow + a.q.stride_h + 16 * kk);
-    }
-    walk_first();
+    MA_TICK(16);
+    walk_first(std::true_type{});
+    MA_TICK(10);
 
     // O^T of both heads: all 256 AGPRs (D = 256); nothing but MFMAs touches them inside the loop
     f32x16 oa[DB], ob[DB];
@@ -285,7 +323,8 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
     pin_tiles<0, DB, true>(ob);
     la = lb = 0.f;
     if (mode != 2) ma_ = mb_ = -INFINITY;
-    if (mode) walk_first();  // a later pass starts the walk again
+    if (mode) walk_first(std::false_type{});  // a later pass starts the walk again
+    MA_TICK(11);
 
     for (int n = 0; have; ++n) {
         MA_TICK(0);
@@ -310,9 +349,10 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
         uint32_t nword = 0;
         // The tile loads of the next step ride in this step's chains, one run every few MFMAs (see
         // kPairPlan): issued in one burst they fill the memory pipeline and stall the wave with the
-        // matrix cores idle.  On the last step of a walk the chains fetch the current tiles once more,
-        // into the free half of the ring: cheaper than a test in every hook.
-        int nlast = min(BN, a.S - ck0) - 1;
+        // matrix cores idle.  On the last step of a walk the chains fetch the first row of the current
+        // tiles over and over (it stays in the L1), into the free half of the ring: cheaper than a test
+        // in every hook.
+        int nlast = 0;
         if (have_next) {
             nword = __builtin_amdgcn_readfirstlane(x0[0]);
             k_at = pair_uniform64(x0[2], x0[3]);
@@ -459,23 +499,27 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
         have = have_next;
     }
 
-    wait_vmem();      // (the chains of the last step have fetched its own tiles once more: no test in the hooks)
+    wait_vmem();      // (the chains of the last step have fetched the first row of its own tiles again: no test in the hooks)
     __syncthreads();  // every wave is done with the K/V buffers, and with the flag
     const int redo = *outgrown;
     if (mode == 0 && redo) { mode = 1; continue; }
     if (mode == 1) { mode = 2; continue; }
     break;
     }  // passes
+    MA_TICK(12);
 
     // Epilogue: O^T (a lane owns one q row, 4 consecutive d per register group) goes through the
     // wave's LDS scratch so that the global stores are whole 16-byte-per-lane row segments.
     __syncthreads();  // every wave is done with the K/V buffers
     mfma_fence();
+    MA_TICK(13);
     {
         constexpr int kPitchO = D * 2 + 16;
         lds_ptr Os = lds0 + w * 32 * kPitchO;
         constexpr int CH = D / 8, RPI = 64 / CH;
         const int rsub = lane / CH, c = lane % CH;
+        const int64_t o_stride_s = a.o.stride_s;
+        const uint32_t o_row_bytes = (uint32_t)(o_stride_s * 2);
         // (one copy of the code per head: picked at run time, every element would be read from both
         // accumulators and selected)
         static_for<0, 2>([&](auto hsel_c) {
@@ -493,15 +537,25 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
                     *(MA_LDS bf16x4*)(Os + r * kPitchO + (32 * db + 8 * g + 4 * hh) * 2) = pk;
                 }
             }
-            __bf16* og = (__bf16*)a.o.ptr + b * a.o.stride_b + (h0 + hsel) * a.o.stride_h;
+            if constexpr (hsel == 0) MA_TICK(18);
+            // all of the wave's rows leave LDS first, then go out: one LDS round trip and no dependent
+            // scalar load per store (the row stride is read once, offsets are 32-bit)
+            MA_GLB char* og = (MA_GLB char*)((__bf16*)a.o.ptr + b * a.o.stride_b + (h0 + hsel) * a.o.stride_h + (int64_t)qw_lo * o_stride_s);
+            u32x4 val[32 / RPI];
 #pragma unroll
-            for (int it = 0; it < 32 / RPI; ++it) {
-                const int row = it * RPI + rsub;
-                const u32x4 val = *(MA_LDS u32x4*)(Os + row * kPitchO + c * 16);
-                if (qw_lo + row < a.S) *(u32x4*)(og + (int64_t)(qw_lo + row) * a.o.stride_s + c * 8) = val;
+            for (int it = 0; it < 32 / RPI; ++it) val[it] = *(MA_LDS u32x4*)(Os + (it * RPI + rsub) * kPitchO + c * 16);
+            if constexpr (hsel == 0) MA_TICK(19);
+            if (qw_lo + 31 < a.S) {
+#pragma unroll
+                for (int it = 0; it < 32 / RPI; ++it) *(MA_GLB u32x4*)(og + (uint32_t)(it * RPI + rsub) * o_row_bytes + c * 16) = val[it];
+            } else {
+#pragma unroll
+                for (int it = 0; it < 32 / RPI; ++it)
+                    if (qw_lo + it * RPI + rsub < a.S) *(MA_GLB u32x4*)(og + (uint32_t)(it * RPI + rsub) * o_row_bytes + c * 16) = val[it];
             }
             if (qvalid && hh == 0)
                 a.lse[((size_t)b * a.Hq + h0 + hsel) * a.S + q] = l > 0.f ? (m + __log2f(l)) * kLn2 : -INFINITY;
+            if constexpr (hsel == 0) { MA_TICK(14); } else { MA_TICK(15); }
         });
     }
 }
