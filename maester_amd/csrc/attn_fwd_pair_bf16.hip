@@ -275,6 +275,16 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
     auto load_ids = [&](uint64_t doc_at, int r0) {
         if (HAS_DOC) kd_next = ((const MA_GLB int64_t*)doc_at)[min(lane, a.S - 1 - r0)];
     };
+    // O^T of both heads: all 256 AGPRs (D = 256); nothing but MFMAs touches them inside the loop
+    f32x16 oa[DB], ob[DB];
+    auto zero_acc = [&]() {
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) oa[db][v] = ob[db][v] = 0.f;
+        pin_tiles<0, DB, true>(oa);
+        pin_tiles<0, DB, true>(ob);
+    };
     bf16x8 qa[KK], qb[KK];
     const __bf16* qrow = qp + (int64_t)qc * a.q.stride_s + 8 * hh;
     auto load_qa = [&]() {
@@ -284,6 +294,7 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
     auto load_qb = [&]() {
 #pragma unroll
         for (int kk = 0; kk < KK; ++kk) qb[kk] = *(const bf16x8*)(qrow + a.q.stride_h + 16 * kk);
+        zero_acc();  // (while the loads are on their way)
     };
     auto walk_first = [&](auto first_c) {
         st.start((MA_LDS uint32_t*)(lds0 + 4 * TL::bytes(BN) + 2 * BN * 8 + 16) + w * (kPairRecBytes / 4));
@@ -305,9 +316,6 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
     MA_TICK(16);
     walk_first(std::true_type{});
     MA_TICK(10);
-
-    // O^T of both heads: all 256 AGPRs (D = 256); nothing but MFMAs touches them inside the loop
-    f32x16 oa[DB], ob[DB];
     float ma_ = -INFINITY, mb_ = -INFINITY, la = 0.f, lb = 0.f;
     MA_LDS int* outgrown = (MA_LDS int*)(lds0 + 4 * TL::bytes(BN) + 2 * BN * 8);
     if (tid == 0) *outgrown = 0;
@@ -315,15 +323,12 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
 
     // mode 0: the one pass described above; mode 1: row maxima only; mode 2: accumulate against them
     for (int mode = 0;; ) {
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) oa[db][v] = ob[db][v] = 0.f;
-    pin_tiles<0, DB, true>(oa);
-    pin_tiles<0, DB, true>(ob);
     la = lb = 0.f;
     if (mode != 2) ma_ = mb_ = -INFINITY;
-    if (mode) walk_first(std::false_type{});  // a later pass starts the walk again
+    if (mode) {  // a later pass starts the walk again (the first pass cleared the accumulators while its loads were on their way)
+        zero_acc();
+        walk_first(std::false_type{});
+    }
     MA_TICK(11);
 
     for (int n = 0; have; ++n) {
