@@ -10,6 +10,9 @@ measuring at one counter read per mark.  The marks:
     8 item ends              1 behind the step's barrier   3 behind its first chain (S, dP / S^T)
                              6 step ends                   4 before its second chain (dV, dK / O^T)
                                                            5 behind its second chain
+  forward only:  9 the item's place in the schedule is known   10 its first tiles are requested (walk resolved,
+                 Q rows requested)   11 the pass begins   12 the passes are over   13 epilogue begins (behind its
+                 barrier)   14 / 15 first / second head is written out
 
 ``python -m maester_amd.kernel_ticks build`` (no GPU needed) builds one variant library per interval
 into ``maester_amd/ticks_build/``; ``python -m maester_amd.kernel_ticks measure --workload c2`` runs
@@ -38,6 +41,17 @@ INTERVALS = [(0, 1, "step begins -> behind the barrier (rows to LDS, next record
              (7, 0, "item begins -> first step (prologue)"),
              (6, 8, "last step ends -> item ends (epilogue)"),
              (7, 8, "whole item")]
+EXTRA = {"fwd": [(7, 9, "item begins -> its place in the schedule is known (ticket, order entry)"),
+                 (9, 10, "-> walk resolved, Q rows and first tiles requested"),
+                 (10, 11, "-> the pass begins"),
+                 (6, 12, "last step ends -> the passes are over (last wait for the tiles, barrier, redo flag)"),
+                 (13, 14, "epilogue: first head scaled, turned through LDS and written out"),
+                 (14, 15, "epilogue: second head")],
+         "dkv": []}
+
+
+def _intervals(kernel: str):
+    return INTERVALS + EXTRA[kernel]
 
 
 def _variant(kernel: str, a: int, b: int) -> str:
@@ -66,13 +80,13 @@ def build_variants(jobs: int = 6) -> None:
     from concurrent.futures import ThreadPoolExecutor
     os.makedirs(OUT, exist_ok=True)
     _build.build()  # the other objects come from the library's own build
-    todo = [(kernel, src, a, b) for kernel, (src, _) in KERNELS.items() for a, b, _ in INTERVALS]
+    todo = [(kernel, src, a, b) for kernel, (src, _) in KERNELS.items() for a, b, _ in _intervals(kernel)]
     with ThreadPoolExecutor(max_workers=jobs) as ex:
         for path in ex.map(_build_one, todo):
             print("built", path, flush=True)
 
 
-def _one(kernel: str, a: int, b: int, workload: str, launches: int) -> None:
+def _one(kernel: str, a: int, b: int, workload: str, launches: int, settle: float) -> None:
     """Runs in a process of its own: the variant library is the only one this process loads."""
     import torch
     from . import _lib
@@ -95,9 +109,14 @@ def _one(kernel: str, a: int, b: int, workload: str, launches: int) -> None:
         run = lambda: attention_forward(q, k, wl.xv, tm, wl.document_ids, wl.scale, True, sp.window)
     read = getattr(ctypes.CDLL(_lib.LIB_PATH), KERNELS[kernel][1])
     vals = (ctypes.c_ulonglong * 4)()
-    for _ in range(5):
-        run()
-    torch.cuda.synchronize()
+    import time
+    t_end = time.time() + settle  # the clocks climb for a while after the GPU was idle: measure what they settle at
+    while True:
+        for _ in range(10):
+            run()
+        torch.cuda.synchronize()
+        if time.time() >= t_end:
+            break
     read(vals, 1)
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
@@ -112,13 +131,13 @@ def _one(kernel: str, a: int, b: int, workload: str, launches: int) -> None:
           f"the wave's {tot / max(wgs, 1) / 1e3:8.1f} kcycles; {ms:.4f} ms per launch -> {tot / max(wgs, 1) / ms / 1e3:.0f} MHz", flush=True)
 
 
-def measure(workload: str, kernels: list, launches: int) -> None:
+def measure(workload: str, kernels: list, launches: int, settle: float) -> None:
     for kernel in kernels:
-        for a, b, what in INTERVALS:
+        for a, b, what in _intervals(kernel):
             if not os.path.exists(_variant(kernel, a, b)):
                 raise RuntimeError(f"{_variant(kernel, a, b)} is missing: run `python -m maester_amd.kernel_ticks build` first")
             res = subprocess.run([sys.executable, "-m", "maester_amd.kernel_ticks", "one", "--kernel", kernel, "--begin", str(a), "--end", str(b),
-                                  "--workload", workload, "--launches", str(launches)], capture_output=True, text=True, timeout=300)
+                                  "--workload", workload, "--launches", str(launches), "--settle-seconds", str(settle)], capture_output=True, text=True, timeout=300)
             if res.returncode != 0:
                 raise RuntimeError(res.stderr[-2000:])
             print(res.stdout.strip() + f"   # {what}", flush=True)
@@ -132,10 +151,11 @@ if __name__ == "__main__":
     ap.add_argument("--begin", type=int, default=0)
     ap.add_argument("--end", type=int, default=6)
     ap.add_argument("--launches", type=int, default=20)
+    ap.add_argument("--settle-seconds", type=float, default=1.5, help="launches repeated this long before the measured ones")
     args = ap.parse_args()
     if args.what == "build":
         build_variants()
     elif args.what == "measure":
-        measure(args.workload, [args.kernel] if args.kernel else ["fwd", "dkv"], args.launches)
+        measure(args.workload, [args.kernel] if args.kernel else ["fwd", "dkv"], args.launches, args.settle_seconds)
     else:
-        _one(args.kernel, args.begin, args.end, args.workload, args.launches)
+        _one(args.kernel, args.begin, args.end, args.workload, args.launches, args.settle_seconds)
