@@ -194,7 +194,7 @@ __device__ __forceinline__ uint64_t pair_uniform64(uint32_t lo, uint32_t hi) {
     return (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane(lo) | ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane(hi) << 32);
 }
 
-template <int D, bool HAS_DOC>
+template <int D, bool HAS_DOC, bool FULL>
 __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int wg_id
 #ifdef MA_TICKS
     , TicksF& ticks
@@ -242,14 +242,41 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
     using SK = DirectStager<D, BN, NW>;
     constexpr int kPaced = (SK::NL - 1) / NW;
     static_assert(SK::NL == NW * kPaced + 1 && (2 * KK) % kPaced == 0 && 4 * DB == 2 * KK, "tile runs per wave");
-    SK sk;
-    sk.init(w, lane);
-    uint32_t rc_last;  // the left-over run, whichever wave moves it
+    // the lane's byte offset into a K tile and into a V tile for each of its runs (the two tensors may have
+    // different row strides), and for the left-over run of the tile its wave moves
+    uint32_t koff[kPaced], voff[kPaced], off_last;
     {
         int row, chunk;
+#pragma unroll
+        for (int p = 0; p < kPaced; ++p) {
+            SK::slot(w + p * NW, lane, row, chunk);
+            koff[p] = (uint32_t)row * ksb + (uint32_t)chunk * 16u;
+            voff[p] = (uint32_t)row * vsb + (uint32_t)chunk * 16u;
+        }
         SK::slot(SK::NL - 1, lane, row, chunk);
-        rc_last = (uint32_t)(row << 16 | chunk * 16);
+        off_last = (uint32_t)row * (w == 0 ? ksb : vsb) + (uint32_t)chunk * 16u;
     }
+    constexpr uint32_t kRowBytes = D * 2;
+    // Where a run comes from.  FULL (the sequence is a whole number of tiles, so every tile has all of its
+    // rows): the tile's address, and a run is a plain load into LDS -- on the last step of a walk, when there
+    // is no next tile, the address stays on the current one, which is read once more.  Otherwise: a buffer
+    // descriptor of the tile with `rows` rows in range; lanes of rows past it (all of them when there is no
+    // next tile) read nothing and zeros land in LDS.  (The plain load is the faster instruction here.)
+    struct Src { uint64_t at; u32x4 rsrc; };
+    auto k_tile = [&](uint64_t at, int rows) {
+        Src t{at, u32x4{0, 0, 0, 0}};
+        if constexpr (!FULL) t.rsrc = tile_rsrc(at, rows > 0 ? (uint32_t)(rows - 1) * ksb + kRowBytes : 0u);
+        return t;
+    };
+    auto v_tile = [&](uint64_t at, int rows) {
+        Src t{at, u32x4{0, 0, 0, 0}};
+        if constexpr (!FULL) t.rsrc = tile_rsrc(at, rows > 0 ? (uint32_t)(rows - 1) * vsb + kRowBytes : 0u);
+        return t;
+    };
+    auto run_to_lds = [&](const Src& t, uint32_t off, uint32_t lds) {
+        if constexpr (FULL) global_to_lds_run((const void*)t.at, off, lds);
+        else buffer_to_lds_run(t.rsrc, off, lds);
+    };
     int64_t kd_next = 0;
 
     // The walk over the kv tiles: its index loads go out first, then both heads' Q rows, which go
@@ -308,8 +335,13 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
             k_at = pair_uniform64(x0[2], x0[3]);
             v_at = pair_uniform64(x1[0], x1[1]);
             const int rows_valid = min(BN, a.S - k0);
-            sk.issue((const __bf16*)k_at, Kbuf(0), w, lane, rows_valid, a.k.stride_s);
-            sk.issue((const __bf16*)v_at, Vbuf(0), w, lane, rows_valid, a.v.stride_s);
+            const Src kr = k_tile(k_at, rows_valid), vr = v_tile(v_at, rows_valid);
+#pragma unroll
+            for (int p = 0; p < kPaced; ++p) run_to_lds(kr, koff[p], lds_addr(Kbuf(0)) + (w + p * NW) * 1024);
+            if (w == 0) run_to_lds(kr, off_last, lds_addr(Kbuf(0)) + (SK::NL - 1) * 1024);
+#pragma unroll
+            for (int p = 0; p < kPaced; ++p) run_to_lds(vr, voff[p], lds_addr(Vbuf(0)) + (w + p * NW) * 1024);
+            if (w == 1) run_to_lds(vr, off_last, lds_addr(Vbuf(0)) + (SK::NL - 1) * 1024);
             load_ids(pair_uniform64(x1[2], x1[3]), k0);
         }
     };
@@ -354,19 +386,22 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
         uint32_t nword = 0;
         // The tile loads of the next step ride in this step's chains, one run every few MFMAs (see
         // kPairPlan): issued in one burst they fill the memory pipeline and stall the wave with the
-        // matrix cores idle.  On the last step of a walk the chains fetch the first row of the current
-        // tiles over and over (it stays in the L1), into the free half of the ring: cheaper than a test
-        // in every hook.
-        int nlast = 0;
+        // matrix cores idle.  On the last step of a walk the loads stay in the chains -- cheaper than a test
+        // in every hook -- and fill the free half of the ring with the current tiles once more, or with zeros
+        // (see run_to_lds).
+        int nrows = 0;
         if (have_next) {
             nword = __builtin_amdgcn_readfirstlane(x0[0]);
             k_at = pair_uniform64(x0[2], x0[3]);
             v_at = pair_uniform64(x1[0], x1[1]);
             const int nk0 = (int)(nword & 0xffffffu);
             load_ids(pair_uniform64(x1[2], x1[3]), nk0);
-            nlast = min(BN, a.S - nk0) - 1;
-            if (w == 0) global_to_lds_run_rc((const void*)k_at, rc_last, ksb, nlast, lds_addr(Kbuf(cur ^ 1)) + (SK::NL - 1) * 1024);
-            if (w == 1 && mode != 1) global_to_lds_run_rc((const void*)v_at, rc_last, vsb, nlast, lds_addr(Vbuf(cur ^ 1)) + (SK::NL - 1) * 1024);
+            nrows = min(BN, a.S - nk0);
+        }
+        const Src kr = k_tile(k_at, nrows), vr = v_tile(v_at, nrows);
+        if (have_next) {
+            if (w == 0) run_to_lds(kr, off_last, lds_addr(Kbuf(cur ^ 1)) + (SK::NL - 1) * 1024);
+            if (w == 1 && mode != 1) run_to_lds(vr, off_last, lds_addr(Vbuf(cur ^ 1)) + (SK::NL - 1) * 1024);
         }
         const uint32_t kdst = lds_addr(Kbuf(cur ^ 1)), vdst = lds_addr(Vbuf(cur ^ 1));
 
@@ -388,9 +423,9 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
             auto move_run = [&](auto tile_c, auto run_c) {
                 constexpr int run = decltype(run_c)::value;
                 if constexpr (decltype(tile_c)::value == 0)
-                    global_to_lds_run_rc((const void*)k_at, sk.rc[run], ksb, nlast, kdst + w * 1024 + run * (NW * 1024));
+                    run_to_lds(kr, koff[run], kdst + w * 1024 + run * (NW * 1024));
                 else
-                    global_to_lds_run_rc((const void*)v_at, sk.rc[run], vsb, nlast, vdst + w * 1024 + run * (NW * 1024));
+                    run_to_lds(vr, voff[run], vdst + w * 1024 + run * (NW * 1024));
             };
             auto burst_plan = [&](auto plan_c) {
                 constexpr int which = decltype(plan_c)::value;
@@ -504,7 +539,7 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
         have = have_next;
     }
 
-    wait_vmem();      // (the chains of the last step have fetched the first row of its own tiles again: no test in the hooks)
+    wait_vmem();      // (the chains of the last step have written to the free half of the ring)
     __syncthreads();  // every wave is done with the K/V buffers, and with the flag
     const int redo = *outgrown;
     if (mode == 0 && redo) { mode = 1; continue; }
@@ -567,7 +602,7 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
 
 // One workgroup per work item, or -- with work queues in the tile map -- one per compute unit, pulling
 // items until none is left (see WorkQueue).
-template <int D, bool HAS_DOC>
+template <int D, bool HAS_DOC, bool FULL>
 __global__ __launch_bounds__(kPairThreads) void attn_fwd_pair_bf16_kernel(AttnArgs a) {
     extern __shared__ __align__(16) char smem_raw[];
     MA_LDS int* box = (MA_LDS int*)((lds_ptr)smem_raw + (4 * Tile<D>::bytes(kPairBN) + 2 * kPairBN * 8 + 4));
@@ -578,7 +613,7 @@ __global__ __launch_bounds__(kPairThreads) void attn_fwd_pair_bf16_kernel(AttnAr
     const unsigned long long t_start = __builtin_readcyclecounter();
     for (int id = wq.next(box); id >= 0; id = wq.next(box)) {
         MA_TICK(7);
-        attn_fwd_pair_bf16_item<D, HAS_DOC>(fresh_args(), id, ticks);
+        attn_fwd_pair_bf16_item<D, HAS_DOC, FULL>(fresh_args(), id, ticks);
         __syncthreads();
         MA_TICK(8);
     }
@@ -590,34 +625,42 @@ __global__ __launch_bounds__(kPairThreads) void attn_fwd_pair_bf16_kernel(AttnAr
     }
 #else
     for (int id = wq.next(box); id >= 0; id = wq.next(box)) {
-        attn_fwd_pair_bf16_item<D, HAS_DOC>(fresh_args(), id);
+        attn_fwd_pair_bf16_item<D, HAS_DOC, FULL>(fresh_args(), id);
         __syncthreads();  // the item's LDS (and the box) are free again
     }
 #endif
     wq.leave();
 }
 
-template <int D, bool HAS_DOC>
+template <int D, bool HAS_DOC, bool FULL>
 static int pair_dd(const AttnArgs& a, hipStream_t st) {
     const size_t lds = (size_t)4 * Tile<D>::bytes(kPairBN) + 2 * kPairBN * 8 + 16 + (kPairThreads / 64) * kPairRecBytes;  // K/V ring, kv ids, redo flag + work-queue box, step records
     if (lds > 64 * 1024) {
-        hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_pair_bf16_kernel<D, HAS_DOC>,
+        hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_pair_bf16_kernel<D, HAS_DOC, FULL>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return fail(MA_ERR_LAUNCH, "hipFuncSetAttribute(attn_fwd_pair_bf16, %zu): %s", lds, hipGetErrorString(e));
     }
     const int GP = a.Hq / a.Hkv / 2;
-    static const int resident = resident_workgroups(attn_fwd_pair_bf16_kernel<D, HAS_DOC>, kPairThreads, lds);
-    hipLaunchKernelGGL((attn_fwd_pair_bf16_kernel<D, HAS_DOC>), dim3(queue_grid(work_grid(a.B * a.T, a.Hkv, GP), a.map.work_counters, resident), 1, 1),
+    static const int resident = resident_workgroups(attn_fwd_pair_bf16_kernel<D, HAS_DOC, FULL>, kPairThreads, lds);
+    hipLaunchKernelGGL((attn_fwd_pair_bf16_kernel<D, HAS_DOC, FULL>), dim3(queue_grid(work_grid(a.B * a.T, a.Hkv, GP), a.map.work_counters, resident), 1, 1),
                        dim3(kPairThreads), lds, st, a);
     return check_launch("attn_fwd_pair_bf16_kernel");
 }
 
 // Only for head layouts with an even number of query heads per kv head; the caller checks.
+template <int D>
+static int pair_d(const AttnArgs& a, hipStream_t st) {
+    // every tile has all of its rows when the sequence is a whole number of kv steps
+    const bool full = a.S % kPairBN == 0;
+    if (a.doc) return full ? pair_dd<D, true, true>(a, st) : pair_dd<D, true, false>(a, st);
+    return full ? pair_dd<D, false, true>(a, st) : pair_dd<D, false, false>(a, st);
+}
+
 int launch_attn_fwd_pair_bf16(const AttnArgs& a, hipStream_t st) {
     switch (a.D) {
-        case 64: return a.doc ? pair_dd<64, true>(a, st) : pair_dd<64, false>(a, st);
-        case 128: return a.doc ? pair_dd<128, true>(a, st) : pair_dd<128, false>(a, st);
-        case 256: return a.doc ? pair_dd<256, true>(a, st) : pair_dd<256, false>(a, st);
+        case 64: return pair_d<64>(a, st);
+        case 128: return pair_d<128>(a, st);
+        case 256: return pair_d<256>(a, st);
     }
     return fail(MA_ERR_UNSUPPORTED, "attn_fwd bf16: head_dim %d not in {64,128,256}", a.D);
 }
