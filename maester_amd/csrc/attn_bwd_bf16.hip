@@ -277,7 +277,7 @@ __device__ __forceinline__ uint64_t uniform64(uint32_t lo, uint32_t hi) {
 
 // WRITE_DS: every 32 x 32 block of every step the workgroup walks also leaves its dS^T in a.ds (zeros
 // for a block the wave skips), for the dQ kernel that only multiplies it with K.
-template <int D, bool HAS_DOC, bool WRITE_DS>
+template <int D, bool HAS_DOC, bool WRITE_DS, bool FULL>
 __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg_id
 #ifdef MA_TICKS
     , Ticks& ticks
@@ -350,20 +350,42 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
     using SQ = DirectStager<D, BM, NW>;
     constexpr int kPaced = (SQ::NL - 1) / NW;
     static_assert(SQ::NL == NW * kPaced + 1 && (2 * KK) % kPaced == 0, "tile runs per wave");
-    SQ sq;
-    sq.init(w, lane);
-    uint32_t rc_last;  // the left-over run, whichever wave moves it
+    const uint32_t qsb = (uint32_t)(a.q.stride_s * 2), gsb = (uint32_t)(a.dout.stride_s * 2);  // row strides in bytes
+    // the lane's byte offset into a Q tile and into a dO tile for each of its runs (the two tensors may have
+    // different row strides), and for the left-over run of the tile its wave moves
+    uint32_t qoff[kPaced], goff[kPaced], off_last;
     {
         int row, chunk;
-        SQ::slot(SQ::NL - 1, lane, row, chunk);
-        rc_last = (uint32_t)(row << 16 | chunk * 16);
-    }
-    const uint32_t qsb = (uint32_t)(a.q.stride_s * 2), gsb = (uint32_t)(a.dout.stride_s * 2);  // row strides in bytes
-    // a whole tile at once (the first step of an item, and a block this wave skips)
-    auto burst = [&](const void* src, uint32_t dst, uint32_t stride_bytes, int last_row, bool with_last) {
 #pragma unroll
-        for (int p = 0; p < kPaced; ++p) global_to_lds_run_rc(src, sq.rc[p], stride_bytes, last_row, dst + (w + p * NW) * 1024);
-        if (with_last) global_to_lds_run_rc(src, rc_last, stride_bytes, last_row, dst + (SQ::NL - 1) * 1024);
+        for (int p = 0; p < kPaced; ++p) {
+            SQ::slot(w + p * NW, lane, row, chunk);
+            qoff[p] = (uint32_t)row * qsb + (uint32_t)chunk * 16u;
+            goff[p] = (uint32_t)row * gsb + (uint32_t)chunk * 16u;
+        }
+        SQ::slot(SQ::NL - 1, lane, row, chunk);
+        off_last = (uint32_t)row * (w == 0 ? qsb : gsb) + (uint32_t)chunk * 16u;
+    }
+    constexpr uint32_t kRowBytes = D * 2;
+    // Where a run comes from.  FULL (the sequence is a whole number of steps, so every tile has all of its
+    // rows): the tile's address, and a run is a plain load into LDS -- on the last step of a walk, when there
+    // is no next tile, the address stays on the current one, which is read once more.  Otherwise: a buffer
+    // descriptor of the tile with `rows` rows in range; lanes of rows past it (all of them when there is no
+    // next tile) read nothing and zeros land in LDS.  (The plain load is the faster instruction here.)
+    struct Src { uint64_t at; u32x4 rsrc; };
+    auto tile_src = [&](uint64_t at, int rows, uint32_t stride_bytes) {
+        Src t{at, u32x4{0, 0, 0, 0}};
+        if constexpr (!FULL) t.rsrc = tile_rsrc(at, rows > 0 ? (uint32_t)(rows - 1) * stride_bytes + kRowBytes : 0u);
+        return t;
+    };
+    auto run_to_lds = [&](const Src& t, uint32_t off, uint32_t lds) {
+        if constexpr (FULL) global_to_lds_run((const void*)t.at, off, lds);
+        else buffer_to_lds_run(t.rsrc, off, lds);
+    };
+    // a whole tile at once (the first step of an item)
+    auto burst = [&](const Src& t, const uint32_t* off, uint32_t dst, bool with_last) {
+#pragma unroll
+        for (int p = 0; p < kPaced; ++p) run_to_lds(t, off[p], dst + (w + p * NW) * 1024);
+        if (with_last) run_to_lds(t, off_last, dst + (SQ::NL - 1) * 1024);
     };
     // per-row lse / delta / document id of a step: loaded for the step after the current one, written
     // to LDS when that step begins by wave 1 (lse), wave 2 (delta) and wave 3 (ids).  Every wave issues
@@ -401,9 +423,9 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
         ds_at = uniform64(x2[2], x2[3]);
         decode(flags);
         const int r0 = q0;
-        const int last = min(BM, S - r0) - 1;
-        burst((const void*)nq_at, lds_addr(Qbuf(0)), qsb, last, w == 0);
-        burst((const void*)ng_at, lds_addr(Gbuf(0)), gsb, last, w == 1);
+        const int rows = min(BM, S - r0);
+        burst(tile_src(nq_at, rows, qsb), qoff, lds_addr(Qbuf(0)), w == 0);
+        burst(tile_src(ng_at, rows, gsb), goff, lds_addr(Gbuf(0)), w == 1);
         load_rows(uniform64(x1[2], x1[3]), uniform64(x2[0], x2[1]), r0);
     }
     const uint32_t ds_lane = (uint32_t)((32 * w + r) * (kTile * 2) + 16 * hh);
@@ -438,17 +460,20 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
         // one run every four MFMAs (Q tile from the S / dP chain, dO tile from the dV / dK chain): issued
         // in one burst they fill the memory pipeline and stall the wave with the matrix cores idle, and
         // issued later in the step they have not landed when the next step begins.
-        int nlast = 0;  // (the last step of a walk: its chains fetch the first row of the current tiles again, see below)
+        int nrows = 0;  // (the last step of a walk: see run_to_lds)
         if (have_next) {
             nflags = __builtin_amdgcn_readfirstlane(x0[0]);
             nq_at = uniform64(x0[2], x0[3]);
             ng_at = uniform64(x1[0], x1[1]);
             nds_at = uniform64(x2[2], x2[3]);
             const int nr0 = (int)(nflags & 0xffffffu);
-            nlast = min(BM, S - nr0) - 1;
+            nrows = min(BM, S - nr0);
             load_rows(uniform64(x1[2], x1[3]), uniform64(x2[0], x2[1]), nr0);
-            if (w == 0) global_to_lds_run_rc((const void*)nq_at, rc_last, qsb, nlast, lds_addr(Qbuf(cur ^ 1)) + (SQ::NL - 1) * 1024);
-            if (w == 1) global_to_lds_run_rc((const void*)ng_at, rc_last, gsb, nlast, lds_addr(Gbuf(cur ^ 1)) + (SQ::NL - 1) * 1024);
+        }
+        const Src qsrc = tile_src(nq_at, nrows, qsb), gsrc = tile_src(ng_at, nrows, gsb);
+        if (have_next) {
+            if (w == 0) run_to_lds(qsrc, off_last, lds_addr(Qbuf(cur ^ 1)) + (SQ::NL - 1) * 1024);
+            if (w == 1) run_to_lds(gsrc, off_last, lds_addr(Gbuf(cur ^ 1)) + (SQ::NL - 1) * 1024);
         }
         const uint32_t qdst = lds_addr(Qbuf(cur ^ 1)), gdst = lds_addr(Gbuf(cur ^ 1));
 
@@ -464,9 +489,9 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
             auto move_run = [&](auto tile_c, auto run_c) {
                 constexpr int run = decltype(run_c)::value;
                 if constexpr (decltype(tile_c)::value == 0)
-                    global_to_lds_run_rc((const void*)nq_at, sq.rc[run], qsb, nlast, qdst + w * 1024 + run * (NW * 1024));
+                    run_to_lds(qsrc, qoff[run], qdst + w * 1024 + run * (NW * 1024));
                 else
-                    global_to_lds_run_rc((const void*)ng_at, sq.rc[run], gsb, nlast, gdst + w * 1024 + run * (NW * 1024));
+                    run_to_lds(gsrc, goff[run], gdst + w * 1024 + run * (NW * 1024));
             };
             if (skip[mb]) {
                 if (WRITE_DS) {
@@ -595,8 +620,7 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
         have = have_next;
     }
 
-    wait_vmem();      // (the chains of the last step have fetched the first row of its own tiles over and over, into the
-                      // free half of the ring: no test in the hooks, and nothing that leaves the L1)
+    wait_vmem();      // (the chains of the last step have written to the free half of the ring: no test in the hooks)
     __syncthreads();  // everyone is done with the tiles: reuse the ring as store scratch
     mfma_fence();
     {
@@ -611,7 +635,7 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
 
 // One workgroup per work item, or -- with work queues in the tile map -- one per compute unit, pulling
 // items until none is left (see WorkQueue).
-template <int D, bool HAS_DOC, bool WRITE_DS>
+template <int D, bool HAS_DOC, bool WRITE_DS, bool FULL>
 __global__ __launch_bounds__(kBwdThreads, D <= 128 ? MA_DKV_WAVES : 1) void attn_bwd_dkv_bf16_kernel(AttnArgs a) {
     extern __shared__ __align__(16) char smem_raw[];
     MA_LDS int* box = (MA_LDS int*)((lds_ptr)smem_raw + (4 * Tile<D>::bytes(kStep) + 2 * kStep * (4 + 4 + 8)));
@@ -622,7 +646,7 @@ __global__ __launch_bounds__(kBwdThreads, D <= 128 ? MA_DKV_WAVES : 1) void attn
     const unsigned long long t_start = __builtin_readcyclecounter();
     for (int id = wq.next(box); id >= 0; id = wq.next(box)) {
         MA_TICK(7);
-        attn_bwd_dkv_bf16_item<D, HAS_DOC, WRITE_DS>(fresh_args(), id, ticks);
+        attn_bwd_dkv_bf16_item<D, HAS_DOC, WRITE_DS, FULL>(fresh_args(), id, ticks);
         __syncthreads();
         MA_TICK(8);
     }
@@ -634,7 +658,7 @@ __global__ __launch_bounds__(kBwdThreads, D <= 128 ? MA_DKV_WAVES : 1) void attn
     }
 #else
     for (int id = wq.next(box); id >= 0; id = wq.next(box)) {
-        attn_bwd_dkv_bf16_item<D, HAS_DOC, WRITE_DS>(fresh_args(), id);
+        attn_bwd_dkv_bf16_item<D, HAS_DOC, WRITE_DS, FULL>(fresh_args(), id);
         __syncthreads();  // the item's LDS (and the box) are free again
     }
 #endif
@@ -1157,6 +1181,17 @@ static int opt_in_lds(K kernel, size_t bytes, const char* name) {
     return MA_OK;
 }
 
+// FULL: every q step of the sequence has all of its rows (see the kernel's run_to_lds)
+template <int D, bool HAS_DOC, bool WRITE_DS, bool FULL>
+static int launch_dkv(const AttnArgs& a, size_t lds_kv, hipStream_t st) {
+    int rc = opt_in_lds(attn_bwd_dkv_bf16_kernel<D, HAS_DOC, WRITE_DS, FULL>, lds_kv, "attn_bwd_dkv_bf16");
+    if (rc) return rc;
+    static const int resident = resident_workgroups(attn_bwd_dkv_bf16_kernel<D, HAS_DOC, WRITE_DS, FULL>, kBwdThreads, lds_kv);
+    hipLaunchKernelGGL((attn_bwd_dkv_bf16_kernel<D, HAS_DOC, WRITE_DS, FULL>), dim3(queue_grid(work_grid(a.B * a.T, a.Hkv, 1), a.map.work_counters, resident), 1, 1),
+                       dim3(kBwdThreads), lds_kv, st, a);
+    return check_launch("attn_bwd_dkv_bf16_kernel");
+}
+
 template <int D, bool HAS_DOC>
 static int bwd_dd(const AttnArgs& a, hipStream_t st) {
     constexpr int RPB = 256 / (D / 8);
@@ -1173,12 +1208,7 @@ static int bwd_dd(const AttnArgs& a, hipStream_t st) {
     const size_t lds_kv = (size_t)4 * Tile<D>::bytes(kStep) + 2 * kStep * (4 + 4 + 8) + 16 + (kBwdThreads / 64) * kDkvRecBytes;  // + work-queue box, step records
     if (hand_over) {
         if (a.stages & MA_BWD_DKV) {
-            rc = opt_in_lds(attn_bwd_dkv_bf16_kernel<D, HAS_DOC, true>, lds_kv, "attn_bwd_dkv_bf16");
-            if (rc) return rc;
-            static const int resident = resident_workgroups(attn_bwd_dkv_bf16_kernel<D, HAS_DOC, true>, kBwdThreads, lds_kv);
-            hipLaunchKernelGGL((attn_bwd_dkv_bf16_kernel<D, HAS_DOC, true>), dim3(queue_grid(work_grid(a.B * a.T, a.Hkv, 1), a.map.work_counters, resident), 1, 1),
-                               dim3(kBwdThreads), lds_kv, st, a);
-            rc = check_launch("attn_bwd_dkv_bf16_kernel");
+            rc = a.S % kStep == 0 ? launch_dkv<D, HAS_DOC, true, true>(a, lds_kv, st) : launch_dkv<D, HAS_DOC, true, false>(a, lds_kv, st);
             if (rc) return rc;
         }
         const int G = a.Hq / a.Hkv;
@@ -1211,12 +1241,7 @@ static int bwd_dd(const AttnArgs& a, hipStream_t st) {
         if (rc) return rc;
     }
     if (a.stages & MA_BWD_DKV) {
-        rc = opt_in_lds(attn_bwd_dkv_bf16_kernel<D, HAS_DOC, false>, lds_kv, "attn_bwd_dkv_bf16");
-        if (rc) return rc;
-        static const int resident = resident_workgroups(attn_bwd_dkv_bf16_kernel<D, HAS_DOC, false>, kBwdThreads, lds_kv);
-        hipLaunchKernelGGL((attn_bwd_dkv_bf16_kernel<D, HAS_DOC, false>), dim3(queue_grid(work_grid(a.B * a.T, a.Hkv, 1), a.map.work_counters, resident), 1, 1), dim3(kBwdThreads), lds_kv,
-                           st, a);
-        rc = check_launch("attn_bwd_dkv_bf16_kernel");
+        rc = a.S % kStep == 0 ? launch_dkv<D, HAS_DOC, false, true>(a, lds_kv, st) : launch_dkv<D, HAS_DOC, false, false>(a, lds_kv, st);
     }
     return rc;
 }
