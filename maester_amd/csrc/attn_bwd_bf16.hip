@@ -381,6 +381,10 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
         if constexpr (FULL) global_to_lds_run((const void*)t.at, off, lds);
         else buffer_to_lds_run(t.rsrc, off, lds);
     };
+    auto run_to_lds_at = [&](const Src& t, uint32_t off, uint32_t lds_base, auto imm_c) {
+        if constexpr (FULL) global_to_lds_run_at<decltype(imm_c)::value>((const void*)t.at, off, lds_base);
+        else buffer_to_lds_run_at<decltype(imm_c)::value>(t.rsrc, off, lds_base);
+    };
     // a whole tile at once (the first step of an item)
     auto burst = [&](const Src& t, const uint32_t* off, uint32_t dst, bool with_last) {
 #pragma unroll
@@ -475,7 +479,7 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
             if (w == 0) run_to_lds(qsrc, off_last, lds_addr(Qbuf(cur ^ 1)) + (SQ::NL - 1) * 1024);
             if (w == 1) run_to_lds(gsrc, off_last, lds_addr(Gbuf(cur ^ 1)) + (SQ::NL - 1) * 1024);
         }
-        const uint32_t qdst = lds_addr(Qbuf(cur ^ 1)), gdst = lds_addr(Gbuf(cur ^ 1));
+        const uint32_t qdst = lds_addr(Qbuf(cur ^ 1)) + w * 1024, gdst = lds_addr(Gbuf(cur ^ 1)) + w * 1024;  // the wave's first run
 
         // The two 32-row blocks of the step are two copies of the same code (mb is a compile-time
         // constant in each), so that each chain carries exactly the loads planned for it.
@@ -489,9 +493,9 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
             auto move_run = [&](auto tile_c, auto run_c) {
                 constexpr int run = decltype(run_c)::value;
                 if constexpr (decltype(tile_c)::value == 0)
-                    run_to_lds(qsrc, qoff[run], qdst + w * 1024 + run * (NW * 1024));
+                    run_to_lds_at(qsrc, qoff[run], qdst, std::integral_constant<int, run * (NW * 1024)>{});
                 else
-                    run_to_lds(gsrc, goff[run], gdst + w * 1024 + run * (NW * 1024));
+                    run_to_lds_at(gsrc, goff[run], gdst, std::integral_constant<int, run * (NW * 1024)>{});
             };
             if (skip[mb]) {
                 if (WRITE_DS) {

@@ -277,6 +277,10 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
         if constexpr (FULL) global_to_lds_run((const void*)t.at, off, lds);
         else buffer_to_lds_run(t.rsrc, off, lds);
     };
+    auto run_to_lds_at = [&](const Src& t, uint32_t off, uint32_t lds_base, auto imm_c) {
+        if constexpr (FULL) global_to_lds_run_at<decltype(imm_c)::value>((const void*)t.at, off, lds_base);
+        else buffer_to_lds_run_at<decltype(imm_c)::value>(t.rsrc, off, lds_base);
+    };
     int64_t kd_next = 0;
 
     // The walk over the kv tiles: its index loads go out first, then both heads' Q rows, which go
@@ -403,7 +407,7 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
             if (w == 0) run_to_lds(kr, off_last, lds_addr(Kbuf(cur ^ 1)) + (SK::NL - 1) * 1024);
             if (w == 1 && mode != 1) run_to_lds(vr, off_last, lds_addr(Vbuf(cur ^ 1)) + (SK::NL - 1) * 1024);
         }
-        const uint32_t kdst = lds_addr(Kbuf(cur ^ 1)), vdst = lds_addr(Vbuf(cur ^ 1));
+        const uint32_t kdst = lds_addr(Kbuf(cur ^ 1)) + w * 1024, vdst = lds_addr(Vbuf(cur ^ 1)) + w * 1024;  // the wave's first run
 
         // mask constants of this step (see attn_fwd_bf16_kernel)
         const int qrel = q - ck0 - 4 * hh;
@@ -423,9 +427,9 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
             auto move_run = [&](auto tile_c, auto run_c) {
                 constexpr int run = decltype(run_c)::value;
                 if constexpr (decltype(tile_c)::value == 0)
-                    run_to_lds(kr, koff[run], kdst + w * 1024 + run * (NW * 1024));
+                    run_to_lds_at(kr, koff[run], kdst, std::integral_constant<int, run * (NW * 1024)>{});
                 else
-                    run_to_lds(vr, voff[run], vdst + w * 1024 + run * (NW * 1024));
+                    run_to_lds_at(vr, voff[run], vdst, std::integral_constant<int, run * (NW * 1024)>{});
             };
             auto burst_plan = [&](auto plan_c) {
                 constexpr int which = decltype(plan_c)::value;

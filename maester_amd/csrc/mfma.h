@@ -514,6 +514,16 @@ __device__ __forceinline__ u32x4 tile_rsrc(uint64_t base, uint32_t bytes_in_rang
     asm volatile("" : "+s"(r));
     return r;
 }
+// (the same two with the LDS address given as a wave-uniform base plus a compile-time constant: the sum goes
+// straight into m0, one instruction less than adding first and moving then)
+template <int IMM>
+__device__ __forceinline__ void global_to_lds_run_at(const void* base, uint32_t voff, uint32_t lds_base) {
+    asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(voff), "s"(base), "n"(IMM) : "m0", "scc");
+}
+template <int IMM>
+__device__ __forceinline__ void buffer_to_lds_run_at(const u32x4 rsrc, uint32_t voff, uint32_t lds_base) {
+    asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_base), "v"(voff), "s"(rsrc), "n"(IMM) : "m0", "scc");
+}
 __device__ __forceinline__ void buffer_to_lds_run(const u32x4 rsrc, uint32_t voff, uint32_t lds) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds), "v"(voff), "s"(rsrc) : "m0");
 }
