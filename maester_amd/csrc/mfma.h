@@ -527,43 +527,6 @@ __device__ __forceinline__ void buffer_to_lds_run_at(const u32x4 rsrc, uint32_t 
 __device__ __forceinline__ void buffer_to_lds_run(const u32x4 rsrc, uint32_t voff, uint32_t lds) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds), "v"(voff), "s"(rsrc) : "m0");
 }
-// The same with the lane's offset worked out on the spot from its packed (source row << 16 | byte offset
-// inside the row): min(row, last_row) * stride_bytes + offset, as part of the asm statement -- left to
-// the compiler, the pieces that do not change from step to step are hoisted out of the loops and cost
-// the kernels registers they do not have.  (The vector instructions between the write of m0 and the
-// load are the wait state the load needs.)
-__device__ __forceinline__ void global_to_lds_run_rc(const void* base, uint32_t rc, uint32_t stride_bytes, int last_row, uint32_t lds) {
-    uint32_t t, u;
-    asm volatile(
-        "s_mov_b32 m0, %[lds]\n\t"
-        "v_lshrrev_b32 %[t], 16, %[rc]\n\t"
-        "v_and_b32 %[u], 0xffff, %[rc]\n\t"
-        "v_min_i32 %[t], %[last], %[t]\n\t"
-        "v_mad_u32_u24 %[t], %[t], %[stride], %[u]\n\t"
-        "global_load_lds_dwordx4 %[t], %[base]"
-        : [t] "=&v"(t), [u] "=&v"(u)
-        : [rc] "v"(rc), [last] "s"(last_row), [stride] "s"(stride_bytes), [lds] "s"(lds), [base] "s"(base)
-        : "m0");
-}
-// The same again, skipped as a whole when the wave-uniform `on` is zero (one compare-and-branch: the
-// hooks of a chain that runs once per 32-row block use it to move their tile in the first block only).
-__device__ __forceinline__ void global_to_lds_run_rc_if(uint32_t on, const void* base, uint32_t rc, uint32_t stride_bytes, int last_row,
-                                                        uint32_t lds) {
-    uint32_t t, u;
-    asm volatile(
-        "s_cmp_eq_u32 %[on], 0\n\t"
-        "s_cbranch_scc1 .Lma_skip_run%=\n\t"
-        "s_mov_b32 m0, %[lds]\n\t"
-        "v_lshrrev_b32 %[t], 16, %[rc]\n\t"
-        "v_and_b32 %[u], 0xffff, %[rc]\n\t"
-        "v_min_i32 %[t], %[last], %[t]\n\t"
-        "v_mad_u32_u24 %[t], %[t], %[stride], %[u]\n\t"
-        "global_load_lds_dwordx4 %[t], %[base]\n"
-        ".Lma_skip_run%=:"
-        : [t] "=&v"(t), [u] "=&v"(u)
-        : [on] "s"(on), [rc] "v"(rc), [last] "s"(last_row), [stride] "s"(stride_bytes), [lds] "s"(lds), [base] "s"(base)
-        : "m0", "scc");
-}
 #pragma clang diagnostic pop
 template <int D, int ROWS, int NWAVES>
 struct DirectStager {

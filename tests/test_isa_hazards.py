@@ -42,8 +42,9 @@ def test_generated_assembly_of_the_attention_kernels_is_hazard_free():
     bad, stats = isa_check.check_all()
     assert not bad, "\n".join(bad[:20])
     # every bf16 attention kernel went through the checker, and its asm MFMAs were seen
-    # (three head dims x with / without document ids; the dK/dV kernel also with / without the dS hand-over)
-    for kernel, count in (("attn_fwd_bf16_kernel", 6), ("attn_fwd_pair_bf16_kernel", 6), ("attn_bwd_dq_bf16_kernel", 6),
-                          ("attn_bwd_dq_ds_bf16_kernel", 6), ("attn_bwd_dkv_bf16_kernel", 12)):
+    # (three head dims x with / without document ids; the pair forward and the dK/dV kernel also with plain or
+    # descriptor tile loads, the dK/dV kernel with / without the dS hand-over)
+    for kernel, count in (("attn_fwd_bf16_kernel", 6), ("attn_fwd_pair_bf16_kernel", 12), ("attn_bwd_dq_bf16_kernel", 6),
+                          ("attn_bwd_dq_ds_bf16_kernel", 6), ("attn_bwd_dkv_bf16_kernel", 24)):
         hits = [v for k, v in stats.items() if kernel in k]
         assert len(hits) == count and all(n_mfma > 0 for n_mfma, _ in hits), (kernel, hits)
