@@ -125,6 +125,7 @@ __global__ __launch_bounds__(256) void attn_delta_bf16_kernel(AttnArgs a) {
 // record of ready-made addresses in the wave's own slice of LDS; taking a step is then three
 // broadcast LDS reads and a dozen v_readfirstlane.
 //   word 0       first q row | query head within the group << 24 | act1 << 29 | act0 << 30 | partial << 31
+//   word 1       rows of the step that lie inside the sequence (1 .. 64)
 //                (act0 / act1: this wave has something to do in the first / second 32-row block)
 //   words 2,3    address of the step's first Q row        words 4,5    of its first dO row
 //   words 6,7    of its first lse entry                   words 8,9    of its first delta entry
@@ -248,7 +249,7 @@ struct DkvSteps {
                 }
                 MA_LDS uint32_t* rec = tab + at * kDkvRecWords;
                 *(MA_LDS u32x4*)rec = u32x4{(uint32_t)r0 | ((uint32_t)rep << 24) | ((uint32_t)act1 << 29) | ((uint32_t)act0 << 30) | ((uint32_t)partial << 31),
-                                            0u, (uint32_t)qa, (uint32_t)(qa >> 32)};
+                                            (uint32_t)min(kStep, a.S - r0), (uint32_t)qa, (uint32_t)(qa >> 32)};
                 *(MA_LDS u32x4*)(rec + 4) = u32x4{(uint32_t)ga, (uint32_t)(ga >> 32), (uint32_t)la, (uint32_t)(la >> 32)};
                 *(MA_LDS u32x4*)(rec + 8) = u32x4{(uint32_t)ea, (uint32_t)(ea >> 32), (uint32_t)da, (uint32_t)(da >> 32)};
             }
@@ -397,8 +398,8 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
     // for on the spot, to merge its result with the value carried otherwise).
     float row_f = 0.f;
     int64_t row_d = 0;
-    auto load_rows = [&](uint64_t lse_at, uint64_t delta_at, int r0) {
-        const int li = min(lane, S - 1 - r0);
+    auto load_rows = [&](uint64_t lse_at, uint64_t delta_at, int r0, int rows) {
+        const int li = min(lane, rows - 1);
         const MA_GLB float* fsrc = (const MA_GLB float*)(w == 2 ? delta_at : lse_at);
         row_f = fsrc[li];
         if (HAS_DOC) row_d = ((const MA_GLB int64_t*)drow)[r0 + li];
@@ -427,10 +428,10 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
         ds_at = uniform64(x2[2], x2[3]);
         decode(flags);
         const int r0 = q0;
-        const int rows = min(BM, S - r0);
+        const int rows = (int)__builtin_amdgcn_readfirstlane(x0[1]);
         burst(tile_src(nq_at, rows, qsb), qoff, lds_addr(Qbuf(0)), w == 0);
         burst(tile_src(ng_at, rows, gsb), goff, lds_addr(Gbuf(0)), w == 1);
-        load_rows(uniform64(x1[2], x1[3]), uniform64(x2[0], x2[1]), r0);
+        load_rows(uniform64(x1[2], x1[3]), uniform64(x2[0], x2[1]), r0, rows);
     }
     const uint32_t ds_lane = (uint32_t)((32 * w + r) * (kTile * 2) + 16 * hh);
 
@@ -471,8 +472,8 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
             ng_at = uniform64(x1[0], x1[1]);
             nds_at = uniform64(x2[2], x2[3]);
             const int nr0 = (int)(nflags & 0xffffffu);
-            nrows = min(BM, S - nr0);
-            load_rows(uniform64(x1[2], x1[3]), uniform64(x2[0], x2[1]), nr0);
+            nrows = (int)__builtin_amdgcn_readfirstlane(x0[1]);  // (from the record: the sequence length is not kept in a register)
+            load_rows(uniform64(x1[2], x1[3]), uniform64(x2[0], x2[1]), nr0, nrows);
         }
         const Src qsrc = tile_src(nq_at, nrows, qsb), gsrc = tile_src(ng_at, nrows, gsb);
         if (have_next) {

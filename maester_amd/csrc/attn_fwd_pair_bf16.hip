@@ -76,6 +76,7 @@ constexpr int kPairPlan[2][2][3] = {{{0, 0, 8}, {0, 0, 0}}, {{0, 0, 0}, {1, 0, 8
 // ready-made addresses in the wave's own slice of LDS; taking a step is then two broadcast LDS reads
 // and a few v_readfirstlane.
 //   word 0       first kv row | act1 << 29 | act0 << 30 | partial << 31
+//   word 1       rows of the step that lie inside the sequence (1 .. 64)
 //                (act0 / act1: this wave has something to do in the first / second 32-row block)
 //   words 2,3    address of the step's first K row        words 4,5    of its first V row
 //   words 6,7    of the document id of its first row (HAS_DOC)
@@ -167,8 +168,8 @@ struct PairSteps {
                 const uint64_t ka = (uint64_t)(kp + (uint64_t)(uint32_t)r0 * ksb), va = (uint64_t)(vp + (uint64_t)(uint32_t)r0 * vsb);
                 const uint64_t da = HAS_DOC ? (uint64_t)(a.doc + (size_t)b * a.S + r0) : 0;
                 MA_LDS uint32_t* rec = tab + at * kPairRecWords;
-                *(MA_LDS u32x4*)rec = u32x4{(uint32_t)r0 | ((uint32_t)act1 << 29) | ((uint32_t)act0 << 30) | ((uint32_t)partial << 31), 0u,
-                                            (uint32_t)ka, (uint32_t)(ka >> 32)};
+                *(MA_LDS u32x4*)rec = u32x4{(uint32_t)r0 | ((uint32_t)act1 << 29) | ((uint32_t)act0 << 30) | ((uint32_t)partial << 31),
+                                            (uint32_t)min(kPairBN, a.S - r0), (uint32_t)ka, (uint32_t)(ka >> 32)};
                 *(MA_LDS u32x4*)(rec + 4) = u32x4{(uint32_t)va, (uint32_t)(va >> 32), (uint32_t)da, (uint32_t)(da >> 32)};
             }
             cbase += 64;
@@ -303,8 +304,8 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
     PairSteps<HAS_DOC> st;
     // document ids of a partial step's kv rows: every wave loads them for the step after the current
     // one (no branch: a conditional load would be waited for on the spot), wave 3 writes them to LDS
-    auto load_ids = [&](uint64_t doc_at, int r0) {
-        if (HAS_DOC) kd_next = ((const MA_GLB int64_t*)doc_at)[min(lane, a.S - 1 - r0)];
+    auto load_ids = [&](uint64_t doc_at, int rows) {
+        if (HAS_DOC) kd_next = ((const MA_GLB int64_t*)doc_at)[min(lane, rows - 1)];
     };
     // O^T of both heads: all 256 AGPRs (D = 256); nothing but MFMAs touches them inside the loop
     f32x16 oa[DB], ob[DB];
@@ -338,7 +339,7 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
             decode(__builtin_amdgcn_readfirstlane(x0[0]));
             k_at = pair_uniform64(x0[2], x0[3]);
             v_at = pair_uniform64(x1[0], x1[1]);
-            const int rows_valid = min(BN, a.S - k0);
+            const int rows_valid = (int)__builtin_amdgcn_readfirstlane(x0[1]);
             const Src kr = k_tile(k_at, rows_valid), vr = v_tile(v_at, rows_valid);
 #pragma unroll
             for (int p = 0; p < kPaced; ++p) run_to_lds(kr, koff[p], lds_addr(Kbuf(0)) + (w + p * NW) * 1024);
@@ -346,7 +347,7 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
 #pragma unroll
             for (int p = 0; p < kPaced; ++p) run_to_lds(vr, voff[p], lds_addr(Vbuf(0)) + (w + p * NW) * 1024);
             if (w == 1) run_to_lds(vr, off_last, lds_addr(Vbuf(0)) + (SK::NL - 1) * 1024);
-            load_ids(pair_uniform64(x1[2], x1[3]), k0);
+            load_ids(pair_uniform64(x1[2], x1[3]), rows_valid);
         }
     };
     MA_TICK(16);
@@ -398,9 +399,8 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
             nword = __builtin_amdgcn_readfirstlane(x0[0]);
             k_at = pair_uniform64(x0[2], x0[3]);
             v_at = pair_uniform64(x1[0], x1[1]);
-            const int nk0 = (int)(nword & 0xffffffu);
-            load_ids(pair_uniform64(x1[2], x1[3]), nk0);
-            nrows = min(BN, a.S - nk0);
+            nrows = (int)__builtin_amdgcn_readfirstlane(x0[1]);  // (from the record: the sequence length is not kept in a register)
+            load_ids(pair_uniform64(x1[2], x1[3]), nrows);
         }
         const Src kr = k_tile(k_at, nrows), vr = v_tile(v_at, nrows);
         if (have_next) {
