@@ -139,6 +139,36 @@ def test_bf16_forward(gpu, case):
     assert max_abs(lse.cpu(), wl) <= 2e-2
 
 
+@pytest.mark.parametrize("S", [1024, 777], ids=["whole_tiles", "ragged"])
+def test_bf16_views_with_different_row_strides(gpu, S):
+    """q, k, v, dO as views into wider buffers, each with a row stride of its own (what the fused qkv projection
+    of model.py:358-364 hands over): bit-identical to the same call on packed copies.  S = 1024 takes the
+    kernels' whole-tile loads, S = 777 the ones that go through a descriptor of the tile."""
+    B, Hq, Hkv, D = 2, 4, 2, 256
+    q, k, v, do = (t.to(gpu) for t in _qkv(B, S, Hq, Hkv, D, torch.bfloat16, 21))
+    ids = _ids(B, S, 22, "docs").to(gpu)
+    scale = D ** -0.5
+
+    def wide(t, extra_heads, at):  # the tensor as heads [at, at + H) of a buffer with extra_heads more heads per row
+        H = t.shape[2]
+        buf = torch.full((B, S, H + extra_heads, D), float("nan"), dtype=t.dtype, device=gpu)
+        buf[:, :, at:at + H] = t
+        return buf[:, :, at:at + H]
+
+    qv, kv, vv, dov = wide(q, 3, 1), wide(k, 1, 0), wide(v, 6, 4), wide(do, 2, 2)
+    assert len({t.stride(1) for t in (qv, kv, vv, dov)}) == 4 and not any(t.is_contiguous() for t in (qv, kv, vv, dov))
+    tm = build_tile_map(ids, B, S, True, None, device=gpu)
+    out_a, lse_a = attention_forward(q, k, v, tm, ids, scale, True, None)
+    out_b, lse_b = attention_forward(qv, kv, vv, tm, ids, scale, True, None)
+    assert torch.equal(out_a, out_b) and torch.equal(lse_a, lse_b)
+    grads_a = attention_backward(q, k, v, out_a, do, lse_a, tm, ids, scale, True, None)
+    grads_b = attention_backward(qv, kv, vv, out_a, dov, lse_a, tm, ids, scale, True, None)
+    for name, a, b in zip(("dq", "dk", "dv"), grads_a, grads_b):
+        assert torch.equal(a, b), name
+    want, _ = A.dense_attention(q.cpu(), k.cpu(), v.cpu(), ids.cpu(), scale, True, None, return_lse=True)
+    _check(out_b, want, torch.bfloat16, ("views", S, "out"), flat=True)
+
+
 @pytest.mark.parametrize("case", BF16_CASES, ids=[c[0] for c in BF16_CASES])
 def test_bf16_backward(gpu, case):
     _, B, S, Hq, Hkv, D, window, kind = case
