@@ -39,6 +39,29 @@ __device__ __forceinline__ void load8<uint16_t>(const uint16_t* p, float* v) {
         v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
     }
 }
+// The same in two halves -- the load, and the conversion of what it returned -- so that a kernel can have
+// the next head's elements on their way while it works on the current one's.
+template <typename T>
+struct Raw8;
+template <>
+struct Raw8<float> {
+    float4 a, b;
+    __device__ __forceinline__ void load(const float* p) { a = *(const float4*)p; b = *(const float4*)(p + 4); }
+    __device__ __forceinline__ void get(float* v) const { v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w; }
+};
+template <>
+struct Raw8<uint16_t> {
+    uint4 a;
+    __device__ __forceinline__ void load(const uint16_t* p) { a = *(const uint4*)p; }
+    __device__ __forceinline__ void get(float* v) const {
+        const uint32_t w[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[2 * i] = __uint_as_float(w[i] << 16);
+            v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+        }
+    }
+};
 template <typename T>
 __device__ __forceinline__ void store8(T* p, const float* v);
 template <>
@@ -84,24 +107,43 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) void prologue_fwd_kernel(
     if (tok >= B * S) return;
     const int b = tok / S, s = tok - b * S;
     const int sub = lane % LPH, hsel = lane / LPH;
+    const int H = Hq + Hkv;
+    // where head h of this token lives (a lane group past the last head re-reads the last one and stores nothing)
+    auto src_of = [&](int h) {
+        const int hc = min(h, H - 1);
+        const bool is_q = hc < Hq;
+        const ma_tensor4& ti = is_q ? qi : ki;
+        return (const T*)ti.ptr + b * ti.stride_b + s * ti.stride_s + (is_q ? hc : hc - Hq) * ti.stride_h;
+    };
+    // The first heads' elements are requested before anything else: the position, and then the table rows
+    // that hang on it, are two dependent round trips the elements do not have to wait behind.  After that
+    // the next heads' elements are always on their way while the current ones are worked on.
+    Raw8<T> r1, r2;
+    {
+        const T* src = src_of(hsel);
+        r1.load(src + sub * 8);
+        r2.load(src + D / 2 + sub * 8);
+    }
     const int64_t p = clamp_pos(pos ? pos[tok] : (int64_t)s, n_pos);
     float c[8], sv[8];
     load8<float>(cs + p * (D / 2) + sub * 8, c);
     load8<float>(sn + p * (D / 2) + sub * 8, sv);
-    const int H = Hq + Hkv;
     for (int h0 = 0; h0 < H; h0 += HPW) {
         const int h = h0 + hsel;
+        float x1[8], x2[8];
+        r1.get(x1);
+        r2.get(x2);
+        if (h0 + HPW < H) {  // (wave-uniform)
+            const T* nsrc = src_of(h + HPW);
+            r1.load(nsrc + sub * 8);
+            r2.load(nsrc + D / 2 + sub * 8);
+        }
         if (h >= H) break;  // whole lane groups drop out together
         const bool is_q = h < Hq;
         const int hh = is_q ? h : h - Hq;
-        const ma_tensor4& ti = is_q ? qi : ki;
         const ma_tensor4& to = is_q ? qo : ko;
         const float* w = is_q ? qw : kw;
-        const T* src = (const T*)ti.ptr + b * ti.stride_b + s * ti.stride_s + hh * ti.stride_h;
         T* dst = (T*)to.ptr + b * to.stride_b + s * to.stride_s + hh * to.stride_h;
-        float x1[8], x2[8];
-        load8<T>(src + sub * 8, x1);
-        load8<T>(src + D / 2 + sub * 8, x2);
         if (w) {
             float ss = 0.f;
 #pragma unroll
@@ -167,37 +209,55 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) void prologue_bwd_kernel(
             for (int i = 0; i < 8; ++i) { gk1[i] += 1.f; gk2[i] += 1.f; }
     }
     const int ntok = B * S;
+    // what a head of a token needs from memory: requested as one group, a head ahead of the arithmetic.
+    // No load hangs on a condition: a lane group past the last head re-reads the last one, and a tensor
+    // without norm weight -- whose forward input and rstd are not passed at all (null) -- reads the incoming
+    // gradient a second time and the cos table instead; those values are never used.
+    Raw8<T> rg1, rg2, rx1, rx2;
+    float rr = 0.f;
+    auto request = [&](int tok, int b, int s, int h) {
+        const int hc = min(h, H - 1);
+        const bool is_q = hc < Hq;
+        const int hh = is_q ? hc : hc - Hq;
+        const ma_tensor4& tx = is_q ? qi : ki;
+        const ma_tensor4& tg = is_q ? dqo : dko;
+        const bool normed = (is_q ? qw : kw) != nullptr;  // then tx and the rstd array are there (checked by the caller)
+        const T* gsrc = (const T*)tg.ptr + b * tg.stride_b + s * tg.stride_s + hh * tg.stride_h;
+        const T* xsrc = normed ? (const T*)tx.ptr + b * tx.stride_b + s * tx.stride_s + hh * tx.stride_h : gsrc;
+        rg1.load(gsrc + sub * 8);
+        rg2.load(gsrc + D / 2 + sub * 8);
+        rx1.load(xsrc + sub * 8);
+        rx2.load(xsrc + D / 2 + sub * 8);
+        rr = *(normed ? (is_q ? q_rstd : k_rstd) + (size_t)tok * (is_q ? Hq : Hkv) + hh : cs);
+    };
     for (int tok = blockIdx.x * kWavesPerBlock + wave; tok < ntok; tok += gridDim.x * kWavesPerBlock) {
         const int b = tok / S, s = tok - b * S;
+        request(tok, b, s, hsel);  // (before the position and the table rows that hang on it)
         const int64_t p = clamp_pos(pos ? pos[tok] : (int64_t)s, n_pos);
         float c[8], sv[8];
         load8<float>(cs + p * (D / 2) + sub * 8, c);
         load8<float>(sn + p * (D / 2) + sub * 8, sv);
         for (int h0 = 0; h0 < H; h0 += HPW) {
             const int h = h0 + hsel;
+            float g1[8], g2[8], x1[8], x2[8], dy1[8], dy2[8];
+            rg1.get(g1);
+            rg2.get(g2);
+            rx1.get(x1);
+            rx2.get(x2);
+            const float r = rr;
+            if (h0 + HPW < H) request(tok, b, s, h + HPW);  // (wave-uniform)
             if (h >= H) break;
             const bool is_q = h < Hq;
             const int hh = is_q ? h : h - Hq;
-            const ma_tensor4& tx = is_q ? qi : ki;
-            const ma_tensor4& tg = is_q ? dqo : dko;
             const ma_tensor4& td = is_q ? dqi : dki;
             const float* w = is_q ? qw : kw;
-            const T* gsrc = (const T*)tg.ptr + b * tg.stride_b + s * tg.stride_s + hh * tg.stride_h;
             T* dst = (T*)td.ptr + b * td.stride_b + s * td.stride_s + hh * td.stride_h;
-            float g1[8], g2[8], dy1[8], dy2[8];
-            load8<T>(gsrc + sub * 8, g1);
-            load8<T>(gsrc + D / 2 + sub * 8, g2);
 #pragma unroll
             for (int i = 0; i < 8; ++i) {  // transpose of the rotation
                 dy1[i] = g1[i] * c[i] + g2[i] * sv[i];
                 dy2[i] = -g1[i] * sv[i] + g2[i] * c[i];
             }
             if (w) {
-                const T* xsrc = (const T*)tx.ptr + b * tx.stride_b + s * tx.stride_s + hh * tx.stride_h;
-                float x1[8], x2[8];
-                load8<T>(xsrc + sub * 8, x1);
-                load8<T>(xsrc + D / 2 + sub * 8, x2);
-                const float r = (is_q ? q_rstd : k_rstd)[(size_t)tok * (is_q ? Hq : Hkv) + hh];
                 float dot = 0.f;
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
