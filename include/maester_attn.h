@@ -44,7 +44,10 @@ extern "C" {
 #define MA_DOC_BLOCK 32 /* rows per entry of ma_tile_map.block_doc_range */
 #define MA_WORK_COUNTERS 64 /* ints in ma_tile_map.work_counters */
 
-/* Library version (major*10000 + minor*100 + patch). */
+/* Version of this header (major*10000 + minor*100 + patch).  It changes whenever a struct or a
+ * signature below changes; ma_version() returns the value the library was built with, and a caller
+ * built against another header must not go on (its ma_tile_map has another layout). */
+#define MA_ABI_VERSION 10200
 int ma_version(void);
 
 /* Message describing the last error returned to the calling thread ("" if none). */
@@ -91,7 +94,10 @@ typedef struct ma_tile_map {
      * indexes the dS workspace with it, which then holds visited tiles only.  Both may be NULL (no dS
      * hand-over).  visited_tiles is the HOST copy of tile_count[0] that sizes that workspace: the
      * caller reads it back once per map (one synchronisation per training step, the map being shared
-     * by all layers), or leaves 0: then the backward recomputes instead of handing dS over. */
+     * by all layers), or leaves 0: then the backward recomputes instead of handing dS over.  It must
+     * be the count of THIS build of the map (read after the build has run, on the build's stream): the
+     * kernels clamp every slot number to visited_tiles - 1, so a stale or too small value cannot make
+     * them touch memory past the workspace, but the gradients of such a call are undefined. */
     int32_t* tile_slot;          /* [B,T,T] */
     int32_t* tile_count;         /* [1] */
     int64_t visited_tiles;       /* host value */

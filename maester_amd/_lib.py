@@ -13,6 +13,7 @@ import torch
 
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libmaester_attn.so")
 
+MA_ABI_VERSION = 10200   # include/maester_attn.h: the struct layouts and signatures bound below
 MA_OK = 0
 MA_ERR_BAD_ARG = -1
 MA_ERR_UNSUPPORTED = -2
@@ -67,6 +68,9 @@ def lib() -> ctypes.CDLL:
     TM = POINTER(MaTileMap)
     L.ma_version.restype = c_int
     L.ma_version.argtypes = []
+    if L.ma_version() != MA_ABI_VERSION:
+        raise RuntimeError(f"{LIB_PATH} was built from header version {L.ma_version()}, this binding is for "
+                           f"{MA_ABI_VERSION}: rebuild the library (python -m maester_amd.build)")
     L.ma_last_error.restype = c_char_p
     L.ma_last_error.argtypes = []
     L.ma_probe_mfma.restype = c_int

@@ -10,6 +10,7 @@ Everything runs in the HIP library; there is no PyTorch fallback.
 """
 from __future__ import annotations
 
+import warnings
 from ctypes import byref
 
 import torch
@@ -133,38 +134,72 @@ def attention_forward(q, k, v, tile_map: TileMap, document_ids, scale, causal=Tr
 
 
 # Largest workspace the backward takes for handing dS from the dK/dV kernel to the dQ kernel (bytes), as a
-# fraction of the memory that is free when it is asked for; above it the dQ kernel recomputes S and dP instead.
+# fraction of the memory that is available when the choice is made; above it the dQ kernel recomputes S and dP.
 DS_WORKSPACE_LIMIT = 64 << 30
 DS_WORKSPACE_FREE_FRACTION = 0.5
+# The two backward paths agree to rounding, not bit for bit, so the choice between them must not move while a
+# run is under way.  ``HAND_OVER_DEFAULT`` True / False fixes it for the process; None decides it ONCE per
+# (device, batch shape) from the memory available at that moment and keeps the decision for every later tile
+# map of that shape (``_HAND_OVER_DECISIONS``).  A decision for the hand-over whose workspace then cannot be
+# allocated is withdrawn for good, with a warning -- never silently and never back and forth.
+HAND_OVER_DEFAULT: bool | None = None
+_HAND_OVER_DECISIONS: dict = {}
+
+
+def _available_bytes(device) -> int:
+    """Memory a new torch allocation can draw on: what the driver reports free plus what torch's caching
+    allocator has reserved but not handed out."""
+    if torch.device(device).type != "cuda":
+        return 0
+    free = torch.cuda.mem_get_info(device)[0]
+    cached = torch.cuda.memory_reserved(device) - torch.cuda.memory_allocated(device)
+    return int(free + max(cached, 0))
+
+
+def decide_hand_over(B, S, Hq, dtype, tile_map: TileMap | None, hand_over=None) -> bool:
+    """Whether ``attention_backward`` hands dS from the dK/dV kernel to the dQ kernel for this tile map.
+    Explicit ``hand_over`` wins, then ``HAND_OVER_DEFAULT``, then the decision already taken for this map or
+    for this (device, B, S, Hq); only the first call for a shape looks at the memory."""
+    if dtype != torch.bfloat16 or tile_map is None or tile_map.tile_slot is None:
+        return False
+    if hand_over is None:
+        hand_over = HAND_OVER_DEFAULT
+    if hand_over is not None:
+        return bool(hand_over)
+    if tile_map._hand_over is not None:
+        return tile_map._hand_over
+    dev = tile_map.tile_slot.device
+    key = (dev.index, B, S, Hq)
+    if key not in _HAND_OVER_DECISIONS:
+        large = _lib.lib().ma_attn_bwd_ds_workspace_bytes(B, S, Hq, tile_map.visited_tiles())
+        ok = 0 < large <= DS_WORKSPACE_LIMIT and large <= DS_WORKSPACE_FREE_FRACTION * _available_bytes(dev)
+        _HAND_OVER_DECISIONS[key] = bool(ok)
+    tile_map._hand_over = _HAND_OVER_DECISIONS[key]
+    return tile_map._hand_over
 
 
 def backward_workspace_bytes(B, S, Hq, Hkv, D, dtype, hand_over=None, tile_map: TileMap | None = None) -> int:
     """Workspace of ``attention_backward``: delta alone, or delta plus one 32 KB dS slot per query head and
-    VISITED tile of ``tile_map`` (bf16 only) when that stays under ``DS_WORKSPACE_LIMIT`` and under
-    ``DS_WORKSPACE_FREE_FRACTION`` of the free device memory; ``hand_over`` True / False forces the choice."""
+    VISITED tile of ``tile_map`` (bf16 only) when the hand-over is taken (``decide_hand_over``)."""
     L = _lib.lib()
     small = L.ma_attn_bwd_workspace_bytes(B, S, Hq, Hkv, D)
-    if hand_over is False or dtype != torch.bfloat16 or tile_map is None or tile_map.tile_slot is None:
+    if not decide_hand_over(B, S, Hq, dtype, tile_map, hand_over):
         return small
     large = L.ma_attn_bwd_ds_workspace_bytes(B, S, Hq, tile_map.visited_tiles())
-    if large == 0:
-        return small
-    if hand_over is None:
-        free = torch.cuda.mem_get_info(tile_map.tile_slot.device)[0] if tile_map.tile_slot.is_cuda else 0
-        if large > DS_WORKSPACE_LIMIT or large > DS_WORKSPACE_FREE_FRACTION * free:
-            return small
-    return large
+    return large if large else small
 
 
 def attention_backward(q, k, v, out, dout, lse, tile_map: TileMap, document_ids, scale, causal=True, window=None,
                        stages=_lib.MA_BWD_ALL, buffers=None, hand_over=None):
     """Returns (dq, dk, dv) as new contiguous [B,S,H,D] tensors.  ``stages`` restricts the call to
     some of its kernels (see ``ma_attn_bwd_stages``); ``buffers`` = (dq, dk, dv, workspace) reuses
-    tensors from an earlier call, which staged calls need.  ``hand_over``: see ``backward_workspace_bytes``."""
+    tensors from an earlier call, which staged calls need.  ``hand_over``: see ``decide_hand_over``.
+    The path the call took is left in ``tile_map.last_backward_path`` ("hand_over" / "recompute")."""
     B, S, Hq, Hkv, D = _check_qkv(q, k, v)
     q, k, v, out, dout = (_rowmajor(t) for t in (q, k, v, out, dout))
     dev = q.device
     L = _lib.lib()
+    small = L.ma_attn_bwd_workspace_bytes(B, S, Hq, Hkv, D)
     if buffers is None:
         dq = torch.empty((B, S, Hq, D), dtype=q.dtype, device=dev)
         dk = torch.empty((B, S, Hkv, D), dtype=q.dtype, device=dev)
@@ -172,8 +207,16 @@ def attention_backward(q, k, v, out, dout, lse, tile_map: TileMap, document_ids,
         ws_bytes = backward_workspace_bytes(B, S, Hq, Hkv, D, q.dtype, hand_over, tile_map)
         try:
             ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
-        except torch.cuda.OutOfMemoryError:      # the dS slots did not fit after all: the small workspace, recompute
-            ws_bytes = backward_workspace_bytes(B, S, Hq, Hkv, D, q.dtype, False)
+        except torch.cuda.OutOfMemoryError:
+            if ws_bytes <= small or hand_over is True or HAND_OVER_DEFAULT is True:
+                raise                            # (an explicit request for the hand-over is not overruled)
+            # the dS slots did not fit after all: withdraw the decision for this shape, for the rest of the process
+            warnings.warn(f"maester_amd: no room for the {ws_bytes >> 20} MiB dS workspace of the attention backward; "
+                          f"B={B} S={S} Hq={Hq} recompute S and dP in the dQ kernel from now on (gradients agree with "
+                          "the hand-over path to rounding, not bit for bit)", RuntimeWarning, stacklevel=2)
+            _HAND_OVER_DECISIONS[(dev.index, B, S, Hq)] = False
+            tile_map._hand_over = False
+            ws_bytes = small
             ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
     else:
         dq, dk, dv, ws = buffers
@@ -189,6 +232,11 @@ def attention_backward(q, k, v, out, dout, lse, tile_map: TileMap, document_ids,
             -1 if window is None else int(window), float(scale), _lib.ptr(ws), ws_bytes,
             _lib.dtype_code(q.dtype), B, S, Hq, Hkv, D, int(stages), _lib.current_stream(dev))
     _lib.check(rc)
+    # (the library takes the hand-over when the map carries the numbering and the workspace holds every visited tile)
+    vis = tile_map._visited or 0
+    took = q.dtype == torch.bfloat16 and tile_map.tile_slot is not None and vis > 0 and \
+        ws_bytes >= L.ma_attn_bwd_ds_workspace_bytes(B, S, Hq, vis)
+    tile_map.last_backward_path = "hand_over" if took else "recompute"
     return dq, dk, dv
 
 

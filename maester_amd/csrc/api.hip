@@ -86,7 +86,7 @@ using namespace ma;
 
 extern "C" {
 
-int ma_version(void) { return 100; }
+int ma_version(void) { return MA_ABI_VERSION; }
 
 const char* ma_last_error(void) { return g_err; }
 

@@ -19,10 +19,6 @@
 #include "common.h"
 #include "mfma.h"
 
-#ifndef MA_DKV_WAVES
-#define MA_DKV_WAVES 1
-#endif
-
 namespace ma {
 
 #ifdef MA_TICKS
@@ -48,10 +44,7 @@ struct Ticks {
 
 constexpr int kBwdThreads = 256;
 constexpr int kStep = 64;   // rows staged per step
-#ifndef MA_BPIPE
-#define MA_BPIPE 4
-#endif
-constexpr int kBPipe = MA_BPIPE;   // LDS fragment reads kept in flight ahead of the MFMAs
+constexpr int kBPipe = 4;   // LDS fragment reads kept in flight ahead of the MFMAs
 
 // O tile epilogue shared by the kernels: a wave holds a 32-row x D fp32 tile transposed in registers
 // (lane (r, hh) owns row r and, per 32-column block, columns 8g + 4hh + e); it is scaled, cast to
@@ -135,21 +128,9 @@ __global__ __launch_bounds__(256) void attn_delta_bf16_kernel(AttnArgs a) {
 // it is derived again from the argument block, so that the step loop holds no registers for it.
 // Which chain of a step carries which of the next step's tile loads, in eighths of a wave's runs:
 // kDkvPlan[block][chain (0: S / dP, 1: dV / dK)] = {tile (0: Q, 1: dO), first eighth, eighths}.
-#ifndef MA_DKV_PLACE
-#define MA_DKV_PLACE 0
-#endif
-#ifndef MA_DKV_EXP_HOOKS
-#define MA_DKV_EXP_HOOKS 1
-#endif
-#if MA_DKV_PLACE == 0
+// The Q tile rides in the first block's S / dP chain, the dO tile in the second block's: both in the first
+// block, or split over more chains, measured slower.
 constexpr int kDkvPlan[2][2][3] = {{{0, 0, 8}, {0, 0, 0}}, {{1, 0, 8}, {0, 0, 0}}};
-#elif MA_DKV_PLACE == 1
-constexpr int kDkvPlan[2][2][3] = {{{0, 0, 8}, {1, 0, 8}}, {{0, 0, 0}, {0, 0, 0}}};
-#elif MA_DKV_PLACE == 2
-constexpr int kDkvPlan[2][2][3] = {{{0, 0, 8}, {1, 0, 4}}, {{1, 4, 4}, {0, 0, 0}}};
-#elif MA_DKV_PLACE == 3
-constexpr int kDkvPlan[2][2][3] = {{{0, 0, 4}, {0, 4, 4}}, {{1, 0, 4}, {1, 4, 4}}};
-#endif
 constexpr int kDkvRecWords = 12;
 constexpr int kDkvRecBytes = 64 * kDkvRecWords * 4;  // LDS per wave
 template <bool HAS_DOC, bool WRITE_DS>
@@ -217,7 +198,9 @@ struct DkvSteps {
             // and the tile's slot in the dS workspace.  Where there is nothing to look up (no range table,
             // a full tile, no step) the range load reads the head of the K tensor and its result is not used.
             uint32_t tslot = 0;
-            if constexpr (WRITE_DS) tslot = (uint32_t)((const MA_GLB int32_t*)a.map.tile_slot)[((int64_t)b * a.T + tile) * a.T + j];
+            // (clamped to the workspace: a count that is stale or too small -- it comes from the host -- must not
+            // turn into a store past the end; the gradients of such a call are undefined, memory is not)
+            if constexpr (WRITE_DS) tslot = min((uint32_t)((const MA_GLB int32_t*)a.map.tile_slot)[((int64_t)b * a.T + tile) * a.T + j], (uint32_t)(a.ds_tiles - 1));
             i64x2 e0 = {0, 0}, e1 = {0, 0};
             bool look = false;
             if constexpr (HAS_DOC) {
@@ -454,6 +437,7 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
             x2 = *(MA_LDS u32x4*)(rec + 8);
         }
         wait_vmem();
+        MA_TICK(20);
         __syncthreads();
         MA_TICK(1);
 
@@ -540,7 +524,6 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
                 }
             }
             const uint32_t roff = (uint32_t)(32 * mb * TL::kPitch);
-#if MA_DKV_EXP_HOOKS
             // The two products run one after the other so that the exponentials of S (a quarter-rate
             // instruction each) are taken in the shadow of the dP MFMAs: one value per MFMA, from the
             // second MFMA after S is complete; what does not fit follows the chain.
@@ -553,11 +536,6 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
             rowfrag_gemm2<D, kBPipe, false, false, decltype(chain_hook)&, true, true>(lds_addr(Qs) + rbase + roff, kf, s, lds_addr(Gs) + rbase + roff, vf, dp, chain_hook);
 #pragma unroll
             for (int v = kHooked; v < 16; ++v) s[v] = fast_exp2(s[v] * sl2);
-#else
-            rowfrag_gemm2<D, kBPipe, false, false, decltype(a_hook)&, false, true>(lds_addr(Qs) + rbase + roff, kf, s, lds_addr(Gs) + rbase + roff, vf, dp, a_hook);
-#pragma unroll
-            for (int v = 0; v < 16; ++v) s[v] = fast_exp2(s[v] * sl2);
-#endif
             MA_TICK(3);
 
             bf16x8 pf[2], dsf[2];
@@ -641,7 +619,7 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
 // One workgroup per work item, or -- with work queues in the tile map -- one per compute unit, pulling
 // items until none is left (see WorkQueue).
 template <int D, bool HAS_DOC, bool WRITE_DS, bool FULL>
-__global__ __launch_bounds__(kBwdThreads, D <= 128 ? MA_DKV_WAVES : 1) void attn_bwd_dkv_bf16_kernel(AttnArgs a) {
+__global__ __launch_bounds__(kBwdThreads, 1) void attn_bwd_dkv_bf16_kernel(AttnArgs a) {
     extern __shared__ __align__(16) char smem_raw[];
     MA_LDS int* box = (MA_LDS int*)((lds_ptr)smem_raw + (4 * Tile<D>::bytes(kStep) + 2 * kStep * (4 + 4 + 8)));
     WorkQueue wq;
@@ -923,9 +901,7 @@ __global__ __launch_bounds__(kBwdThreads, D <= 128 ? 2 : 1) void attn_bwd_dq_bf1
 // ------------------------------------------------------------------------------------------------
 // dQ from the dS^T that the dK/dV kernel left in a.ds
 // ------------------------------------------------------------------------------------------------
-#ifndef MA_DQ_PAIR_MIN_D
-#define MA_DQ_PAIR_MIN_D 64   // head dims from which an even GQA group goes through the two-head kernel
-#endif
+constexpr int kDqPairMinD = 64;   // head dims from which an even GQA group goes through the two-head kernel
 // dQ^T += K^T dS^T and nothing else: no Q / dO / O fragments, no scores, no exponentials.  Per step
 // of 64 kv rows the workgroup stages the K tile and the [64 kv][128 q] slab of dS^T of its q tile;
 // both MFMA operands come from LDS through transposed reads of the same kv rows, so their
@@ -964,7 +940,7 @@ __device__ __forceinline__ void attn_bwd_dq_ds_bf16_item(KernArgs& a, const int 
     const int64_t* rng_row = use_rng ? a.map.block_doc_range + (size_t)b * (2 * ((a.S + 63) / 64)) * 2 : nullptr;
     DocRange own;
     StepTable<BN, true> st;
-    st.numbering(a.map.tile_slot, ((int64_t)b * a.T + i) * a.T, 1);     // tile (i, j) of this batch row, j walked
+    st.numbering(a.map.tile_slot, ((int64_t)b * a.T + i) * a.T, 1, a.ds_tiles);     // tile (i, j) of this batch row, j walked
     {
         int lo, hi;
         visibility_limits(false, i * kTile, i * kTile + kTile - 1, BN, bounded, wlim, windowed, lo, hi);
@@ -1075,7 +1051,7 @@ __device__ __forceinline__ void attn_bwd_dq_ds_pair_bf16_item(KernArgs& a, const
     const int64_t* rng_row = use_rng ? a.map.block_doc_range + (size_t)b * (2 * ((a.S + 63) / 64)) * 2 : nullptr;
     DocRange own;
     StepTable<BN, true> st;
-    st.numbering(a.map.tile_slot, ((int64_t)b * a.T + i) * a.T, 1);     // tile (i, j) of this batch row, j walked
+    st.numbering(a.map.tile_slot, ((int64_t)b * a.T + i) * a.T, 1, a.ds_tiles);     // tile (i, j) of this batch row, j walked
     {
         int lo, hi;
         visibility_limits(false, i * kTile, i * kTile + kTile - 1, BN, bounded, wlim, windowed, lo, hi);
@@ -1217,7 +1193,7 @@ static int bwd_dd(const AttnArgs& a, hipStream_t st) {
             if (rc) return rc;
         }
         const int G = a.Hq / a.Hkv;
-        if ((a.stages & MA_BWD_DQ) && G % 2 == 0 && D >= MA_DQ_PAIR_MIN_D) {
+        if ((a.stages & MA_BWD_DQ) && G % 2 == 0 && D >= kDqPairMinD) {
             const size_t lds_q = (size_t)2 * (Tile<D>::bytes(kStep) + 2 * Tile<kTile>::bytes(kStep)) + 16 + (kBwdThreads / 64) * 512;
             rc = opt_in_lds(attn_bwd_dq_ds_pair_bf16_kernel<D, HAS_DOC>, lds_q, "attn_bwd_dq_ds_pair_bf16");
             if (rc) return rc;

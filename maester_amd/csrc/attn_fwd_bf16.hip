@@ -16,9 +16,7 @@
 #include "common.h"
 #include "mfma.h"
 
-#ifndef MA_PAIR_MIN_D
-#define MA_PAIR_MIN_D 256  /* below that the one-head kernel fits two workgroups per compute unit, which beats sharing K/V fragments */
-#endif
+constexpr int kPairMinD = 256;  // below that the one-head kernel fits two workgroups per compute unit, which beats sharing K/V fragments
 
 namespace ma {
 
@@ -332,7 +330,7 @@ static int fwd_d(const AttnArgs& a, hipStream_t st) {
 
 int launch_attn_fwd_bf16(const AttnArgs& a, hipStream_t st) {
     // query heads that share a kv head are processed in pairs when they come in pairs
-    if ((a.Hq / a.Hkv) % 2 == 0 && a.D >= MA_PAIR_MIN_D) return launch_attn_fwd_pair_bf16(a, st);
+    if ((a.Hq / a.Hkv) % 2 == 0 && a.D >= kPairMinD) return launch_attn_fwd_pair_bf16(a, st);
     switch (a.D) {
         case 64: return fwd_d<64>(a, st);
         case 128: return fwd_d<128>(a, st);

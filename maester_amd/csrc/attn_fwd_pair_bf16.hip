@@ -48,27 +48,13 @@ struct TicksF {
 
 constexpr int kPairThreads = 256;
 constexpr int kPairBN = 64;   // kv rows staged per step
-#ifndef MA_PAIR_PK
-#define MA_PAIR_PK 2
-#define MA_PAIR_PV 2
-#endif
-constexpr int kPairPipeK = MA_PAIR_PK;  // LDS fragment reads in flight ahead of the MFMAs (registers are tight)
-constexpr int kPairPipeV = MA_PAIR_PV;
+constexpr int kPairPipeK = 2;  // LDS fragment reads in flight ahead of the MFMAs (registers are tight)
+constexpr int kPairPipeV = 2;
 // Which chain of a step carries which of the next step's tile loads, in eighths of a wave's runs:
 // kPairPlan[block][chain (0: S^T, 1: O^T)] = {tile (0: K, 1: V), first eighth, eighths}.  K rides in S^T
 // chains only (the pass that only finds row maxima has no O^T chains, and needs no V).
-#ifndef MA_PAIR_PLACE
-#define MA_PAIR_PLACE 1
-#endif
-#if MA_PAIR_PLACE == 0
-constexpr int kPairPlan[2][2][3] = {{{0, 0, 8}, {1, 0, 8}}, {{0, 0, 0}, {0, 0, 0}}};
-#elif MA_PAIR_PLACE == 1
+// (K in the first block's S^T chain, V in the second block's: V in an O^T chain measured slower.)
 constexpr int kPairPlan[2][2][3] = {{{0, 0, 8}, {0, 0, 0}}, {{1, 0, 8}, {0, 0, 0}}};
-#elif MA_PAIR_PLACE == 2
-constexpr int kPairPlan[2][2][3] = {{{0, 0, 8}, {1, 0, 4}}, {{1, 4, 4}, {0, 0, 0}}};
-#elif MA_PAIR_PLACE == 3
-constexpr int kPairPlan[2][2][3] = {{{0, 0, 8}, {0, 0, 0}}, {{0, 0, 0}, {1, 0, 8}}};
-#endif
 
 // The kv steps of one work item, resolved ahead of the loop that runs them.  A wave that has its SIMD to
 // itself pays four cycles for every instruction it issues between two MFMA chains, so whatever a step
@@ -382,6 +368,7 @@ __device__ __forceinline__ void attn_fwd_pair_bf16_item(KernArgs& a, const int w
             x1 = *(MA_LDS u32x4*)(rec + 4);
         }
         wait_vmem();
+        MA_TICK(20);
         __syncthreads();
         MA_TICK(1);
 

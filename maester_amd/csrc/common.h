@@ -352,8 +352,9 @@ struct StepTable {
     int64_t slot_base = 0, slot_stride = 0;
     uint32_t ahead_slot = 0;
     int tile_slot = -1;            // of the current step (SLOTS)
-    __device__ __forceinline__ void numbering(const int32_t* table, int64_t base, int64_t stride) {
-        slot_tab = table; slot_base = base; slot_stride = stride;
+    uint32_t slot_last = 0;        // the last slot of the workspace: numbers are clamped to it (a stale count must not read past the end)
+    __device__ __forceinline__ void numbering(const int32_t* table, int64_t base, int64_t stride, int64_t slots) {
+        slot_tab = table; slot_base = base; slot_stride = stride; slot_last = (uint32_t)(slots - 1);
     }
 
     __device__ __forceinline__ void init(const int32_t* partial_list, int n_partial, const int32_t* full_list, int n_full,
@@ -391,7 +392,7 @@ struct StepTable {
         const int at = __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0));
         if (vis) slot[at] = word;
         if constexpr (SLOTS) {
-            if (vis && slot_tab) slot[64 + at] = (uint32_t)slot_tab[slot_base + (int64_t)tile * slot_stride];
+            if (vis && slot_tab) slot[64 + at] = min((uint32_t)slot_tab[slot_base + (int64_t)tile * slot_stride], slot_last);
         }
         cbase += 64;
         return __builtin_popcountll(mask);

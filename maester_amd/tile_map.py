@@ -46,6 +46,8 @@ class TileMap:
     tile_slot: torch.Tensor | None = None
     tile_count: torch.Tensor | None = None
     _visited: int | None = None
+    _hand_over: bool | None = None   # the backward's choice of path for this map (attention.decide_hand_over)
+    last_backward_path: str | None = None
     _last_stream: object = None      # the torch stream of the last launch that used the work queues
 
     def order_on_current_stream(self, device) -> None:
@@ -76,7 +78,14 @@ class TileMap:
         """Number of visited (partial or full) tiles, read back from the device on first use (one
         synchronisation per map; the map of a training step is shared by all layers) and kept."""
         if self._visited is None:
-            self._visited = int(self.tile_count.item()) if self.tile_count is not None else 0
+            if self.tile_count is None:
+                self._visited = 0
+            else:
+                # the count is written by the build, on the stream the build ran on: wait for THAT stream (the
+                # caller may be on another one, where .item() would read the count before it exists)
+                if self._last_stream is not None and not torch.cuda.is_current_stream_capturing():
+                    self._last_stream.synchronize()
+                self._visited = int(self.tile_count.item())
         return self._visited
 
     @property

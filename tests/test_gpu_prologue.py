@@ -2,7 +2,7 @@
 import pytest
 import torch
 
-from conftest import check_bf16, max_abs, rel_l2
+from conftest import check_bf16, check_bf16_sum, max_abs, rel_l2
 from maester_amd import qk_norm_rope, workloads
 from maester_amd.attention import prologue_forward
 from oracle import prologue as P
@@ -93,8 +93,8 @@ def test_backward(gpu, dtype, D, norm):
             assert rel_l2(a.cpu(), b) < rtol
         elif i < 2:       # activations' gradients: the bar of the path, element by element
             check_bf16(a, b, ("prologue bwd", D, norm, i))
-        else:             # weight gradients are sums over B*S*H rows (values in the tens): relative to their size
-            assert max_abs(a.cpu(), b) <= tol * max(1.0, float(b.abs().max())) and rel_l2(a.cpu(), b) < rtol
+        else:             # weight gradients are sums over B*S*H rows
+            check_bf16_sum(a, b, B * S * (Hq if i == 2 else Hkv), ("prologue bwd weight", D, i))
     # run-to-run determinism of the weight-gradient reduction (no atomics)
     if norm:
         got2 = torch.autograd.grad(qk_norm_rope(hq, hk, hqw, hkw, dev(cos), dev(sin), dev(pos)), [hqw, hkw], [dev(gq), dev(gk)])

@@ -11,7 +11,7 @@ import os
 import pytest
 import torch
 
-from conftest import BF16_MAX_ABS, BF16_ONE_ROUNDING, ROOT, check_bf16
+from conftest import BF16_MAX_ABS, ROOT, bf16_half_ulp, check_bf16
 from maester_amd import build_tile_map, workloads
 from maester_amd.attention import attention_backward, attention_forward
 from oracle import attention as A
@@ -22,9 +22,11 @@ pytestmark = pytest.mark.gpu
 def _numbers(got, want, flat):
     got, want = got.detach().double().cpu(), want.detach().double().cpu()
     err = (got - want).abs()
-    lim = torch.full_like(err, BF16_MAX_ABS) if flat else BF16_MAX_ABS + BF16_ONE_ROUNDING * want.abs()
+    lim = torch.full_like(err, BF16_MAX_ABS) if flat else BF16_MAX_ABS + bf16_half_ulp(want)
+    over = err > BF16_MAX_ABS
     return {"max_abs": float(err.max()), "worst_over_limit": float((err / lim).max()),
-            "rel_l2": float((got - want).norm() / want.norm()), "max_ref": float(want.abs().max())}
+            "rel_l2": float((got - want).norm() / want.norm()), "max_ref": float(want.abs().max()),
+            "over_flat_2e-2": int(over.sum()), "min_ref_over_flat": float(want.abs()[over].min()) if bool(over.any()) else None}
 
 
 @pytest.mark.parametrize("name,B,S", [("c2", 1, 2048), ("c3", 1, 2048), ("c5", 1, 2048)])

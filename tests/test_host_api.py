@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     assert set(names) == set(_lib.EXPORTS), (names, _lib.EXPORTS)
     for n in names:
         assert hasattr(L, n), n
-    assert L.ma_version() >= 100
+    assert L.ma_version() == _lib.MA_ABI_VERSION   # the binding refuses a library built from another header
     assert L.ma_last_error() is not None
 
 
@@ -238,6 +238,35 @@ def test_backward_workspace_choice():
     tm._visited = 8 * 1024 * 1024
     assert L.ma_attn_bwd_ds_workspace_bytes(8, 131072, 8, tm._visited) > A.DS_WORKSPACE_LIMIT
     assert A.backward_workspace_bytes(8, 131072, 8, 4, 256, torch.bfloat16, None, tm) == L.ma_attn_bwd_workspace_bytes(8, 131072, 8, 4, 256)
+
+
+def test_backward_path_is_decided_once_per_shape(monkeypatch):
+    """The two backward paths differ in the last bits, so the choice between them must not follow the free
+    memory from call to call: the first map of a shape decides, later maps inherit, an explicit setting wins."""
+    import torch
+    from maester_amd import attention as A
+    from maester_amd.tile_map import TileMap
+    L = _lib.lib()
+    z = torch.zeros(1, dtype=torch.int32)
+    mk = lambda: TileMap(*([z] * 8), seq_len=8192, causal=True, window=None, tile_slot=z, tile_count=torch.tensor([1698], dtype=torch.int32))
+    small, large = L.ma_attn_bwd_workspace_bytes(4, 8192, 8, 4, 256), L.ma_attn_bwd_ds_workspace_bytes(4, 8192, 8, 1698)
+    monkeypatch.setattr(A, "_HAND_OVER_DECISIONS", {})
+    asked = []
+    monkeypatch.setattr(A, "_available_bytes", lambda dev: asked.append(1) or 10 * large)
+    a = mk()
+    assert A.backward_workspace_bytes(4, 8192, 8, 4, 256, torch.bfloat16, None, a) == large and a._hand_over is True
+    monkeypatch.setattr(A, "_available_bytes", lambda dev: asked.append(1) or 0)          # memory gets tight later on
+    b = mk()
+    assert A.backward_workspace_bytes(4, 8192, 8, 4, 256, torch.bfloat16, None, b) == large and len(asked) == 1
+    assert A.backward_workspace_bytes(4, 8192, 8, 4, 256, torch.bfloat16, None, a) == large
+    assert A.backward_workspace_bytes(4, 8192, 8, 4, 256, torch.bfloat16, False, a) == small   # explicit wins, and is not remembered
+    assert A.backward_workspace_bytes(4, 8192, 8, 4, 256, torch.bfloat16, None, a) == large
+    monkeypatch.setattr(A, "HAND_OVER_DEFAULT", False)
+    assert A.backward_workspace_bytes(4, 8192, 8, 4, 256, torch.bfloat16, None, mk()) == small
+    monkeypatch.setattr(A, "HAND_OVER_DEFAULT", None)
+    c = mk()                                                                               # another shape decides afresh
+    assert A.backward_workspace_bytes(2, 8192, 8, 4, 256, torch.bfloat16, None, c) == L.ma_attn_bwd_workspace_bytes(2, 8192, 8, 4, 256)
+    assert c._hand_over is False and len(asked) == 2
 
 
 def test_text_model_mirrors_reference_parameter_names():
