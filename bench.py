@@ -248,13 +248,14 @@ def main():
     sp = wl.spec
     K, W = args.steps, args.warmup
 
-    if args.calibrate_copy:
-        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
-        dst = torch.empty_like(src)
-        for _ in range(3):
-            dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
+    # A plain 256 MiB device-to-device copy: the rate this GPU moves bytes at when nothing else is asked of it (the
+    # bandwidth roof the kernels' traffic is priced against, beside the published 8 TB/s), and -- under rocprofv3
+    # --pmc -- the reference point that FETCH_SIZE / WRITE_SIZE are scaled by.
+    src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+    dst = torch.empty_like(src)
+    t_copy = time_region(lambda: dst.copy_(src), 3 if args.calibrate_copy else 20, 3)
+    copy_gbps = 2 * src.numel() / (t_copy * 1e-3) / 1e9
+    del src, dst
 
     # ---- tile map (once per training step in the model; timed on its own) -------------------
     tmap = build_tile_map(wl.document_ids, sp.B, sp.S, True, sp.window)
@@ -273,9 +274,11 @@ def main():
     if has_bwd:
         dq, dk, dv = attention_backward(q, k, wl.xv, out, wl.dout, lse, tmap, wl.document_ids, wl.scale, True, sp.window)
         ws_bytes = backward_workspace_bytes(sp.B, sp.S, sp.Hq, sp.Hkv, sp.D, q.dtype, False if args.no_hand_over else None, tmap)
-        hand_over = ws_bytes > _lib.lib().ma_attn_bwd_workspace_bytes(sp.B, sp.S, sp.Hq, sp.Hkv, sp.D) and q.dtype == torch.bfloat16
         ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
         bufs = (dq, dk, dv, ws)
+        # the path the timed calls take is read off a call, not assumed
+        attention_backward(q, k, wl.xv, out, wl.dout, lse, tmap, wl.document_ids, wl.scale, True, sp.window, buffers=bufs)
+        hand_over = tmap.last_backward_path == "hand_over"
 
     def fwd():
         return attention_forward(q, k, wl.xv, tmap, wl.document_ids, wl.scale, True, sp.window)
@@ -309,6 +312,26 @@ def main():
         t_pro_b = time_region(
             lambda: prologue_backward(wl.xq, wl.xk, dq, dk, wl.q_w, wl.k_w, wl.cos, wl.sin, wl.position_ids, q_rstd,
                                       k_rstd), K, W)
+    # The same kernels inside the step: the step is issued as its four launches with an event between them, so
+    # that each kernel finds the caches as the kernel before it left them (a kernel repeated alone finds its own
+    # inputs in the memory-side cache: the delta pass takes 1.6 times as long in the step as alone).
+    in_step = None
+    if has_bwd:
+        stages = [("fwd", fwd), ("delta", lambda: bwd(_lib.MA_BWD_DELTA)), ("dkv", lambda: bwd(_lib.MA_BWD_DKV)),
+                  ("dq", lambda: bwd(_lib.MA_BWD_DQ))] if hand_over else \
+                 [("fwd", fwd), ("dq", lambda: bwd(_lib.MA_BWD_DQ | _lib.MA_BWD_DELTA)), ("dkv", lambda: bwd(_lib.MA_BWD_DKV))]
+        for _ in range(W):
+            step()
+        n_ev = min(K, 50)
+        evs = [_events(len(stages) + 1) for _ in range(n_ev)]
+        for row in evs:
+            row[0].record()
+            for (_, f), e in zip(stages, row[1:]):
+                f()
+                e.record()
+        torch.cuda.synchronize()
+        in_step = {name: sum(row[i].elapsed_time(row[i + 1]) for row in evs) / n_ev for i, (name, _) in enumerate(stages)}
+        in_step["sum_ms"] = sum(in_step.values())
     # the whole autograd Function (prologue + attention, forward + backward), for reference
     t_full = None
     if has_bwd:
@@ -402,29 +425,66 @@ def main():
         return None if ms is None else flops / (ms * 1e-3) / 1e12
 
     base = sp.D * sp.Hq * wl.n_pairs
+    pair = (sp.Hq // sp.Hkv) % 2 == 0
+    fwd_name = "attn_fwd_pair_bf16_kernel" if pair and sp.D >= 256 and sp.dtype == torch.bfloat16 else "attn_fwd_bf16_kernel"
+    dq_name = (("attn_bwd_dq_ds_pair_bf16_kernel" if pair else "attn_bwd_dq_ds_bf16_kernel") if has_bwd and hand_over
+               else "attn_bwd_dq_bf16_kernel")
+    # Algorithmic bytes per launch: every operand and result once (what a kernel with unbounded on-chip memory moves)
+    qb = elt * sp.B * sp.S * sp.Hq * sp.D             # one [B,S,Hq,D] tensor
+    kb = elt * sp.B * sp.S * sp.Hkv * sp.D            # one [B,S,Hkv,D] tensor
+    rowb = 4 * sp.B * sp.Hq * sp.S                    # one fp32 [B,Hq,S] array (lse, delta)
+    dsb = (ws_bytes - rowb if has_bwd and hand_over else 0)   # the dS slots of the visited tiles
     kern = {
-        # query heads that share a kv head go through the pair kernel when they come in pairs
-        ("attn_fwd_pair_bf16_kernel" if (sp.Hq // sp.Hkv) % 2 == 0 and sp.D >= 256 and sp.dtype == torch.bfloat16 else "attn_fwd_bf16_kernel"):
-            {"ms": t_fwd, "algorithmic_flops": 4 * base},
-        "attn_bwd_dkv_bf16_kernel": {"ms": t_dkv, "algorithmic_flops": 6 * base},   # dP, dV, dK
-        (("attn_bwd_dq_ds_pair_bf16_kernel" if (sp.Hq // sp.Hkv) % 2 == 0 else "attn_bwd_dq_ds_bf16_kernel")
-         if has_bwd and hand_over else "attn_bwd_dq_bf16_kernel"):
-            {"ms": t_dq, "algorithmic_flops": 2 * base},                            # dQ
+        fwd_name: {"ms": t_fwd, "algorithmic_flops": 4 * base, "algorithmic_bytes": 2 * qb + 2 * kb + rowb},    # Q, K, V in; O, lse out
+        "attn_bwd_dkv_bf16_kernel": {"ms": t_dkv, "algorithmic_flops": 6 * base,                                  # dP, dV, dK
+                                     "algorithmic_bytes": 2 * qb + 4 * kb + 2 * rowb + dsb},                      # Q, dO, K, V, lse, delta in; dK, dV, dS out
+        dq_name: {"ms": t_dq, "algorithmic_flops": 2 * base,                                                      # dQ
+                  "algorithmic_bytes": (dsb + kb + qb) if has_bwd and hand_over else (3 * qb + 2 * kb + 2 * rowb)},
     }
-    for v in kern.values():
-        v["tflops"] = tf(v["algorithmic_flops"], v["ms"])
-    dom_name = max((n for n in kern if kern[n]["ms"] is not None), key=lambda n: kern[n]["ms"])
-    dom = kern[dom_name]
-    roofline = {
-        "kernel": dom_name, "bound": "mfma", "achieved": dom["tflops"], "peak": PEAK_BF16_DENSE_TFLOPS,
-        "unit": "TFLOP/s", "frac": dom["tflops"] / PEAK_BF16_DENSE_TFLOPS, "traffic": None,
-        "avg_launch_ms": dom["ms"], "algorithmic_flops_per_launch": dom["algorithmic_flops"],
-    }
+    if has_bwd and hand_over:
+        kern["attn_delta_bf16_kernel"] = {"ms": t_delta, "algorithmic_flops": 0, "algorithmic_bytes": 2 * qb + rowb}
     traffic_file = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    counters_file = os.path.join(ROOT, "profiles", "mfma_counters.json")
+    tr, ctr = {}, {}
     if os.path.exists(traffic_file):
         with open(traffic_file) as f:
-            tr = json.load(f)
-        roofline["traffic"] = tr.get(sp.name, {}).get(dom_name)
+            tr = json.load(f).get(sp.name, {})
+    if os.path.exists(counters_file):
+        with open(counters_file) as f:
+            ctr = json.load(f).get(sp.name, {})
+    step_name = {fwd_name: "fwd", "attn_bwd_dkv_bf16_kernel": "dkv", dq_name: "dq", "attn_delta_bf16_kernel": "delta"}
+    for n, v in kern.items():
+        if v["ms"] is None:
+            continue
+        v["tflops"] = tf(v["algorithmic_flops"], v["ms"])
+        v["frac_mfma_peak"] = v["tflops"] / PEAK_BF16_DENSE_TFLOPS
+        v["algorithmic_gbps"] = v["algorithmic_bytes"] / (v["ms"] * 1e-3) / 1e9
+        v["frac_hbm_peak"] = v["algorithmic_gbps"] / PEAK_HBM_GBPS
+        v["in_step_ms"] = None if in_step is None else in_step.get(step_name[n])
+        # measured HBM traffic of a launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, calibrated, from profiles/) against
+        # this run's time and this run's copy rate
+        v["traffic_bytes"] = tr.get(n)
+        if v["traffic_bytes"]:
+            v["traffic_gbps"] = v["traffic_bytes"] / (v["ms"] * 1e-3) / 1e9
+            v["traffic_frac_of_copy_rate"] = v["traffic_gbps"] / copy_gbps
+            v["traffic_over_algorithmic"] = v["traffic_bytes"] / v["algorithmic_bytes"]
+        if n in ctr:       # rocprofv3 --pmc counters of the same kernel and workload (profiles/*_mfma_counters.md)
+            v["rocprof"] = ctr[n]
+    timed = [n for n in kern if kern[n]["ms"] is not None and kern[n]["algorithmic_flops"]]
+    dom_name = max(timed, key=lambda n: kern[n]["ms"])
+    dom = kern[dom_name]
+    # the dominant kernel against both roofs, labelled by the one it is nearer to
+    roofs = {"mfma": {"achieved": dom["tflops"], "peak": PEAK_BF16_DENSE_TFLOPS, "unit": "TFLOP/s", "frac": dom["frac_mfma_peak"]},
+             "hbm": {"achieved": dom["algorithmic_gbps"], "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": dom["frac_hbm_peak"]}}
+    bound = max(roofs, key=lambda r: roofs[r]["frac"])
+    roofline = {
+        "kernel": dom_name, "bound": bound, **roofs[bound], "traffic": dom.get("traffic_bytes"),
+        "avg_launch_ms": dom["ms"], "algorithmic_flops_per_launch": dom["algorithmic_flops"],
+        "algorithmic_bytes_per_launch": dom["algorithmic_bytes"], "roofs": roofs,
+        "copy_gbps_this_run": copy_gbps, "traffic_gbps": dom.get("traffic_gbps"),
+        "traffic_frac_of_copy_rate": dom.get("traffic_frac_of_copy_rate"),
+        "mfma_utilisation_rocprof": (dom.get("rocprof") or {}).get("mfma_busy"),
+    }
 
     T = (sp.S + 127) // 128
     n_partial, n_full = int(tmap.kv_num_blocks.sum()), int(tmap.full_kv_num_blocks.sum())
@@ -435,12 +495,15 @@ def main():
         "dtype": "bf16" if sp.dtype == torch.bfloat16 else "f32", "data": "synthetic",
         "config": {"workload": sp.name, "description": sp.description, "B": sp.B, "S": sp.S, "Hq": sp.Hq,
                    "Hkv": sp.Hkv, "D": sp.D, "window": sp.window, "n_pairs": wl.n_pairs,
-                   "timed_region": "ma_attn_fwd + ma_attn_bwd (delta, dK/dV with dS hand-over, dQ) per step, inputs resident in HBM",
+                   "timed_region": ("ma_attn_fwd + ma_attn_bwd (delta, dK/dV with dS hand-over, dQ) per step" if has_bwd and hand_over else
+                                    "ma_attn_fwd + ma_attn_bwd (dQ with delta, dK/dV, both recomputing S and dP) per step" if has_bwd else
+                                    "ma_attn_fwd per step") + ", inputs resident in HBM",
                    "launch": launch},
         "hip_graph_replay": {"ms_per_step": graph_ms_per_step, "error": graph_error,
                              "value": None if graph_ms_per_step is None else total_flops / (graph_ms_per_step * 1e-3) / 1e12},
         "pct_of_bf16_dense_peak": 100.0 * value / PEAK_BF16_DENSE_TFLOPS,
         "peak_bf16_dense_tflops": PEAK_BF16_DENSE_TFLOPS, "peak_hbm_gbps": PEAK_HBM_GBPS,
+        "device_copy_gbps": copy_gbps,
         "settle_seconds": args.settle_seconds,
         "device": props.name, "gcn_arch": getattr(props, "gcnArchName", ""), "cus": props.multi_processor_count,
         "clock_mhz": clock_after, "clock_source": "pp_dpm_sclk right after the timed region (None: not readable on this box)",
@@ -449,7 +512,8 @@ def main():
         "bwd": None if not has_bwd else {"ms": t_bwd, "tflops": tf(fl["bwd"], t_bwd),
                                          "pct_peak": 100 * tf(fl["bwd"], t_bwd) / PEAK_BF16_DENSE_TFLOPS,
                                          "delta_ms": t_delta, "dkv_ms": t_dkv, "dq_ms": t_dq,
-                                         "ds_hand_over": bool(hand_over), "workspace_bytes": int(ws_bytes)},
+                                         "ds_hand_over": bool(hand_over), "path_taken": tmap.last_backward_path,
+                                         "workspace_bytes": int(ws_bytes), "in_step_ms": in_step},
         "fwd_bwd_flashattn_convention_tflops": tf(fl["fwd_bwd_flashattn_convention"], ms_per_step) if has_bwd else None,
         "kernels": kern,
         "prologue": {"fwd_ms": t_pro_f, "fwd_gbps": pro_bytes / (t_pro_f * 1e-3) / 1e9,
