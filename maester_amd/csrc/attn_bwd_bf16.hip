@@ -86,27 +86,38 @@ __device__ __forceinline__ void store_tile_T(lds_ptr scratch, const f32x16* acc,
 // ------------------------------------------------------------------------------------------------
 // delta[b,h,q] = sum_d O[b,q,h,d] * dO[b,q,h,d]
 // ------------------------------------------------------------------------------------------------
+// A pure read stream (O and dO once, 2 * elt * B*S*Hq*D bytes): every thread has the loads of kDeltaRows rows
+// in flight before it adds anything up.
+constexpr int kDeltaRows = 4;
 template <int D>
 __global__ __launch_bounds__(256) void attn_delta_bf16_kernel(AttnArgs a) {
     constexpr int LPR = D / 8;  // lanes per row
     constexpr int RPB = 256 / LPR;
-    const int64_t row = (int64_t)blockIdx.x * RPB + threadIdx.x / LPR;
     const int sub = threadIdx.x % LPR;
     const int64_t nrows = (int64_t)a.B * a.Hq * a.S;
-    float acc = 0.f;
-    if (row < nrows) {
+    const int64_t row0 = (int64_t)blockIdx.x * (RPB * kDeltaRows) + threadIdx.x / LPR;
+    bf16x8 x[kDeltaRows], y[kDeltaRows];
+#pragma unroll
+    for (int i = 0; i < kDeltaRows; ++i) {
+        const int64_t row = min(row0 + i * RPB, nrows - 1);      // (rows past the end re-read the last one; not written)
         const int q = row % a.S;
         const int h = (row / a.S) % a.Hq;
         const int b = row / ((int64_t)a.S * a.Hq);
         const __bf16* op = (const __bf16*)a.o.ptr + b * a.o.stride_b + (int64_t)q * a.o.stride_s + h * a.o.stride_h;
         const __bf16* gp = (const __bf16*)a.dout.ptr + b * a.dout.stride_b + (int64_t)q * a.dout.stride_s + h * a.dout.stride_h;
-        const bf16x8 x = *(const bf16x8*)(op + sub * 8), y = *(const bf16x8*)(gp + sub * 8);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc += (float)x[e] * (float)y[e];
+        x[i] = __builtin_nontemporal_load((const bf16x8*)(op + sub * 8));   // O is not read again in this step (dO is, at once)
+        y[i] = *(const bf16x8*)(gp + sub * 8);
     }
 #pragma unroll
-    for (int off = LPR / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
-    if (row < nrows && sub == 0) a.delta[row] = acc;
+    for (int i = 0; i < kDeltaRows; ++i) {
+        float acc = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc += (float)x[i][e] * (float)y[i][e];
+#pragma unroll
+        for (int off = LPR / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+        const int64_t row = row0 + i * RPB;
+        if (row < nrows && sub == 0) a.delta[row] = acc;
+    }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -901,6 +912,9 @@ __global__ __launch_bounds__(kBwdThreads, D <= 128 ? 2 : 1) void attn_bwd_dq_bf1
 // ------------------------------------------------------------------------------------------------
 // dQ from the dS^T that the dK/dV kernel left in a.ds
 // ------------------------------------------------------------------------------------------------
+// dS^T is read exactly once, by the workgroup that owns its q tile: its loads carry the non-temporal hint, so that
+// they do not displace the K tiles that the workgroups of a document share (dQ -2.5 % on the Gemma-3-4B shape)
+constexpr bool kDsReadOnce = true;
 constexpr int kDqPairMinD = 64;   // head dims from which an even GQA group goes through the two-head kernel
 // dQ^T += K^T dS^T and nothing else: no Q / dO / O fragments, no scores, no exponentials.  Per step
 // of 64 kv rows the workgroup stages the K tile and the [64 kv][128 q] slab of dS^T of its q tile;
@@ -968,7 +982,7 @@ __device__ __forceinline__ void attn_bwd_dq_ds_bf16_item(KernArgs& a, const int 
     const uint32_t ksb = (uint32_t)(a.k.stride_s * 2);
     auto issue = [&](int buf) {  // K rows r0 .. r0+63 and the matching 64 rows of dS^T (row r0 of the tile list = kv row)
         sk.issue((const __bf16*)((const char*)kp + (uint64_t)(uint32_t)st.r0 * ksb), Kbuf(buf), w, lane, min(BN, a.S - st.r0), a.k.stride_s);
-        ss.issue(sp + (size_t)(uint32_t)st.tile_slot * (kTile * kTile) + (size_t)(st.r0 & (kTile - 1)) * kTile, Sbuf(buf), w, lane, BN, kTile);   // the step's 64 kv rows inside its tile's slot
+        ss.template issue<kDsReadOnce>(sp + (size_t)(uint32_t)st.tile_slot * (kTile * kTile) + (size_t)(st.r0 & (kTile - 1)) * kTile, Sbuf(buf), w, lane, BN, kTile);   // the step's 64 kv rows inside its tile's slot
     };
     bool have = st.next();
     bool act0 = st.act0, act1 = st.act1;
@@ -1080,8 +1094,8 @@ __device__ __forceinline__ void attn_bwd_dq_ds_pair_bf16_item(KernArgs& a, const
     auto issue = [&](int buf) {
         sk.issue((const __bf16*)((const char*)kp + (uint64_t)(uint32_t)st.r0 * ksb), Kbuf(buf), w, lane, min(BN, a.S - st.r0), a.k.stride_s);
         const size_t at = (size_t)(uint32_t)st.tile_slot * (kTile * kTile) + (size_t)(st.r0 & (kTile - 1)) * kTile;
-        ss.issue(sp0 + at, Sbuf(buf, 0), w, lane, BN, kTile);
-        ss.issue(sp1 + at, Sbuf(buf, 1), w, lane, BN, kTile);
+        ss.template issue<kDsReadOnce>(sp0 + at, Sbuf(buf, 0), w, lane, BN, kTile);
+        ss.template issue<kDsReadOnce>(sp1 + at, Sbuf(buf, 1), w, lane, BN, kTile);
     };
     const int k_runs = decltype(sk)::runs_of(w), s_runs = decltype(ss)::runs_of(w);
     bool have = st.next();
@@ -1129,9 +1143,9 @@ __device__ __forceinline__ void attn_bwd_dq_ds_pair_bf16_item(KernArgs& a, const
                     if constexpr (nb == 0) {
                         sk.template issue_one<run>(ksrc, kdst, w, k_lim, ksb);
                     } else if constexpr (run < decltype(ss)::PER) {
-                        ss.template issue_one<run>(s0src, s0dst, w, s_lim, kTile * 2);
+                        ss.template issue_one<run, kDsReadOnce>(s0src, s0dst, w, s_lim, kTile * 2);
                     } else {
-                        ss.template issue_one<run - decltype(ss)::PER>(s1src, s1dst, w, s_lim, kTile * 2);
+                        ss.template issue_one<run - decltype(ss)::PER, kDsReadOnce>(s1src, s1dst, w, s_lim, kTile * 2);
                     }
                 }
             };
@@ -1182,7 +1196,7 @@ static int bwd_dd(const AttnArgs& a, hipStream_t st) {
     // delta on its own when the dQ stage, which computes it for its own rows, is not asked for, and
     // always with the hand-over (its dQ kernel reads neither O nor dO)
     if ((a.stages & MA_BWD_DELTA) && (hand_over || !(a.stages & MA_BWD_DQ))) {
-        hipLaunchKernelGGL(attn_delta_bf16_kernel<D>, dim3((unsigned)((nrows + RPB - 1) / RPB)), dim3(256), 0, st, a);
+        hipLaunchKernelGGL(attn_delta_bf16_kernel<D>, dim3((unsigned)((nrows + RPB * kDeltaRows - 1) / (RPB * kDeltaRows))), dim3(256), 0, st, a);
         rc = check_launch("attn_delta_bf16_kernel");
         if (rc) return rc;
     }

@@ -498,6 +498,10 @@ struct Stager {
 __device__ __forceinline__ void global_to_lds_run(const void* base, uint32_t voff, uint32_t lds) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds), "v"(voff), "s"(base) : "m0");
 }
+// the same with the non-temporal hint: for data that is read exactly once (it does not displace what other workgroups share)
+__device__ __forceinline__ void global_to_lds_run_nt(const void* base, uint32_t voff, uint32_t lds) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(lds), "v"(voff), "s"(base) : "m0");
+}
 // The same through a buffer descriptor: the lane's byte offset into the tile is a ready-made register
 // (row * row stride + offset inside the row, the same for every tile of one tensor), and rows past the
 // end of the tile are out of the descriptor's range: such lanes touch no memory and zeros land in LDS.
@@ -561,21 +565,27 @@ struct DirectStager {
         return (uint32_t)min((int)(rc[p] >> 16), last_row) * stride_bytes + (rc[p] & 0xffffu);
     }
     // run P of this wave for a whole tile (all ROWS rows valid), if P < limit (wave-uniform)
-    template <int P>
+    template <int P, bool NT = false>
     __device__ __forceinline__ void issue_one(const __bf16* g, uint32_t tile_addr, int w, int limit, uint32_t stride_bytes) const {
         if constexpr (P < PER) {
-            if (P < limit)
-                global_to_lds_run(g, (rc[P] >> 16) * stride_bytes + (rc[P] & 0xffffu), tile_addr + (w + P * NWAVES) * 1024);
+            if (P < limit) {
+                if constexpr (NT) global_to_lds_run_nt(g, (rc[P] >> 16) * stride_bytes + (rc[P] & 0xffffu), tile_addr + (w + P * NWAVES) * 1024);
+                else global_to_lds_run(g, (rc[P] >> 16) * stride_bytes + (rc[P] & 0xffffu), tile_addr + (w + P * NWAVES) * 1024);
+            }
         }
     }
     // the whole tile at once; rows at or beyond rows_valid re-read the last valid row
+    template <bool NT = false>
     __device__ __forceinline__ void issue(const __bf16* g, lds_ptr tile, int w, int lane, int rows_valid,
                                           int64_t stride) const {
         const uint32_t sb = (uint32_t)(stride * 2);
         const int runs = runs_of(w);
 #pragma unroll
         for (int p = 0; p < PER; ++p)
-            if (p < runs) global_to_lds_run(g, offset(p, sb, rows_valid - 1), lds_addr(tile) + (w + p * NWAVES) * 1024);
+            if (p < runs) {
+                if constexpr (NT) global_to_lds_run_nt(g, offset(p, sb, rows_valid - 1), lds_addr(tile) + (w + p * NWAVES) * 1024);
+                else global_to_lds_run(g, offset(p, sb, rows_valid - 1), lds_addr(tile) + (w + p * NWAVES) * 1024);
+            }
     }
 };
 
