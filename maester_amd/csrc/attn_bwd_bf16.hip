@@ -270,8 +270,13 @@ __device__ __forceinline__ uint64_t uniform64(uint32_t lo, uint32_t hi) {
     return (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane(lo) | ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane(hi) << 32);
 }
 
-// WRITE_DS: every 32 x 32 block of every step the workgroup walks also leaves its dS^T in a.ds (zeros
-// for a block the wave skips), for the dQ kernel that only multiplies it with K.
+// WRITE_DS: every 32 x 32 block that a wave works on also leaves its dS^T in a.ds, for the dQ kernel that only
+// multiplies it with K.  A block that the wave skips is not written, and the dQ kernel never uses it: both
+// kernels decide per 32 x 32 block (32 q rows of one wave there, 32 kv rows of one wave here) by the same three
+// tests -- the tile is partial and (a) the largest q row lies below the smallest kv row, or (b) the smallest q row
+// lies more than the window above the largest kv row, or (c) the document-id ranges of the two row blocks
+// (block_doc_range) are disjoint -- so a block is skipped on both sides or on neither.  (Blocks of q rows past the
+// end of the sequence are skipped here only; there the dQ kernel computes columns that it never stores.)
 template <int D, bool HAS_DOC, bool WRITE_DS, bool FULL>
 __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg_id
 #ifdef MA_TICKS
@@ -494,10 +499,8 @@ __device__ __forceinline__ void attn_bwd_dkv_bf16_item(KernArgs& a, const int wg
                     run_to_lds_at(gsrc, goff[run], gdst, std::integral_constant<int, run * (NW * 1024)>{});
             };
             if (skip[mb]) {
-                if (WRITE_DS) {
-#pragma unroll
-                    for (int pr = 0; pr < 2; ++pr) *(MA_GLB u32x4*)(ds_out + ds_lane + 64 * mb + 32 * pr) = u32x4{0, 0, 0, 0};
-                }
+                // (nothing is left in the dS workspace for a block the wave skips: the dQ kernel skips the same
+                // 32 x 32 blocks -- see the note on WRITE_DS above the kernel)
                 if (have_next) {  // the loads its chains would have carried
                     static_for<0, kPlanA[2]>([&](auto r) { move_run(std::integral_constant<int, kPlanA[0]>{}, std::integral_constant<int, kPlanA[1] + decltype(r)::value>{}); });
                     static_for<0, kPlanB[2]>([&](auto r) { move_run(std::integral_constant<int, kPlanB[0]>{}, std::integral_constant<int, kPlanB[1] + decltype(r)::value>{}); });
@@ -919,9 +922,9 @@ constexpr int kDqPairMinD = 64;   // head dims from which an even GQA group goes
 // dQ^T += K^T dS^T and nothing else: no Q / dO / O fragments, no scores, no exponentials.  Per step
 // of 64 kv rows the workgroup stages the K tile and the [64 kv][128 q] slab of dS^T of its q tile;
 // both MFMA operands come from LDS through transposed reads of the same kv rows, so their
-// contraction orders agree by construction.  Every block this kernel reads has been written: it
-// walks the same tile lists as the dK/dV kernel, that kernel writes all blocks of every step it
-// walks, and a block that can hold a visible pair lies inside a step with a visible pair.
+// contraction orders agree by construction.  Every 32 x 32 block this kernel multiplies has been written: the
+// dK/dV kernel walks the transposed tile lists and skips a block by the same tests as this kernel does (see
+// WRITE_DS there); the slabs are staged whole, and what lies in the blocks nobody wrote is never used.
 template <int D, bool HAS_DOC>
 __device__ __forceinline__ void attn_bwd_dq_ds_bf16_item(KernArgs& a, const int wg_id) {
     using TL = Tile<D>;
