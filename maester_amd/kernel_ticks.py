@@ -7,9 +7,9 @@ marks ``a`` and ``b`` and sums the differences per wave; one interval per build 
 measuring at one counter read per mark.  The marks:
 
     7 item begins            0 step begins                 2 a 32-row block begins
-    8 item ends              1 behind the step's barrier   3 behind its first chain (S, dP / S^T)
-                             6 step ends                   4 before its second chain (dV, dK / O^T)
-                                                           5 behind its second chain
+    8 item ends              20 own tile loads have landed 3 behind its first chain (S, dP / S^T)
+                             1 behind the step's barrier   4 before its second chain (dV, dK / O^T)
+                             6 step ends                   5 behind its second chain
   forward only:  9 the item's place in the schedule is known   10 its first tiles are requested (walk resolved,
                  Q rows requested)   11 the pass begins   12 the passes are over   13 epilogue begins (behind its
                  barrier)   14 / 15 first / second head is written out
@@ -18,6 +18,9 @@ measuring at one counter read per mark.  The marks:
 into ``maester_amd/ticks_build/``; ``python -m maester_amd.kernel_ticks measure --workload c2`` runs
 them on the GPU, each in a process of its own, and prints one line per interval: mean cycles, how
 often per workgroup, share of the wave's cycles, and the clock the kernel ran at (cycles / time).
+``--wave N`` (both commands) measures wave N of every workgroup instead of wave 0: the waves of a
+workgroup skip different 32-row blocks of a partial tile, so what one wave spends at the step's
+barrier (20 -> 1) is mostly the work another wave still has.
 """
 from __future__ import annotations
 
@@ -33,6 +36,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 OUT = os.path.join(HERE, "ticks_build")
 KERNELS = {"dkv": ("attn_bwd_bf16.hip", "ma_dbg_read_ticks"), "fwd": ("attn_fwd_pair_bf16.hip", "ma_dbg_read_ticks_fwd")}
 INTERVALS = [(0, 1, "step begins -> behind the barrier (rows to LDS, next record, wait for the tiles)"),
+             (0, 20, "step begins -> the wave's own tile loads have landed"),
+             (20, 1, "-> behind the barrier (the other waves' loads and work)"),
              (1, 2, "behind the barrier -> first block (control)"),
              (2, 3, "block begins -> behind the first chain"),
              (3, 4, "elementwise between the chains"),
@@ -54,16 +59,19 @@ def _intervals(kernel: str):
     return INTERVALS + EXTRA[kernel]
 
 
+WAVE = 0     # the wave of every workgroup that is measured (set from --wave)
+
+
 def _variant(kernel: str, a: int, b: int) -> str:
-    return os.path.join(OUT, f"libticks_{kernel}_{a}_{b}.so")
+    return os.path.join(OUT, f"libticks_{kernel}_{a}_{b}" + (f"_w{WAVE}" if WAVE else "") + ".so")
 
 
 def _build_one(job) -> str:
     kernel, src, a, b = job
     others = [os.path.join(_build.OBJ_DIR, os.path.splitext(s)[0] + ".o") for s in _build.SOURCES if s != src]
-    obj = os.path.join(OUT, f"{kernel}_{a}_{b}.o")
+    obj = os.path.join(OUT, f"{kernel}_{a}_{b}_w{WAVE}.o")
     flags = [f for f in _build.HIPCC_FLAGS if not f.startswith("-W")]
-    cmd = [_build._hipcc(), *flags, "-DMA_TICKS", f"-DMA_T_BEGIN={a}", f"-DMA_T_END={b}", "-DMA_T_WAVE=0", "-c",
+    cmd = [_build._hipcc(), *flags, "-DMA_TICKS", f"-DMA_T_BEGIN={a}", f"-DMA_T_END={b}", f"-DMA_T_WAVE={WAVE}", "-c",
            os.path.join(_build.CSRC, src), "-o", obj]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
@@ -137,7 +145,7 @@ def measure(workload: str, kernels: list, launches: int, settle: float) -> None:
             if not os.path.exists(_variant(kernel, a, b)):
                 raise RuntimeError(f"{_variant(kernel, a, b)} is missing: run `python -m maester_amd.kernel_ticks build` first")
             res = subprocess.run([sys.executable, "-m", "maester_amd.kernel_ticks", "one", "--kernel", kernel, "--begin", str(a), "--end", str(b),
-                                  "--workload", workload, "--launches", str(launches), "--settle-seconds", str(settle)], capture_output=True, text=True, timeout=300)
+                                  "--wave", str(WAVE), "--workload", workload, "--launches", str(launches), "--settle-seconds", str(settle)], capture_output=True, text=True, timeout=300)
             if res.returncode != 0:
                 raise RuntimeError(res.stderr[-2000:])
             print(res.stdout.strip() + f"   # {what}", flush=True)
@@ -151,8 +159,10 @@ if __name__ == "__main__":
     ap.add_argument("--begin", type=int, default=0)
     ap.add_argument("--end", type=int, default=6)
     ap.add_argument("--launches", type=int, default=20)
+    ap.add_argument("--wave", type=int, default=0, choices=[0, 1, 2, 3], help="which wave of every workgroup is measured")
     ap.add_argument("--settle-seconds", type=float, default=1.5, help="launches repeated this long before the measured ones")
     args = ap.parse_args()
+    WAVE = args.wave
     if args.what == "build":
         build_variants()
     elif args.what == "measure":
