@@ -244,7 +244,8 @@ int ma_attn_fwd(const ma_tensor4* q, const ma_tensor4* k, const ma_tensor4* v, c
  * the dQ kernel reduces to dQ = scale * dS K instead of recomputing S and dO V^T: the same dK and dV
  * up to the summation order of delta, the same dQ up to the rounding of dS to bf16 (which both
  * variants do before the product), fewer MFMAs, for Hq * visited_tiles * 32 KB (0.45 GB at B=4,
- * S=8192, Hq=8 with documents of some hundred tokens).  Nothing in the workspace needs initialising. */
+ * S=8192, Hq=8 with documents of some hundred tokens).  Nothing in the workspace needs initialising:
+ * inside a slot only the 32 x 32 blocks that hold a visible pair are written, and only those are used. */
 size_t ma_attn_bwd_workspace_bytes(int B, int S, int Hq, int Hkv, int D);
 size_t ma_attn_bwd_ds_workspace_bytes(int B, int S, int Hq, int64_t visited_tiles);
 int ma_attn_bwd(const ma_tensor4* q, const ma_tensor4* k, const ma_tensor4* v, const ma_tensor4* out,
