@@ -114,6 +114,26 @@ def check_assembly(asm: str) -> tuple[list[str], dict]:
     return bad, stats
 
 
+def kernel_resources(asm: str) -> dict:
+    """{kernel: {"vgpr", "agpr", "sgpr", "vgpr_spill", "sgpr_spill", "lds"}} from the metadata the compiler
+    appends to its assembly.  The MFMA kernels are written around the register file (accumulators that fill
+    all 256 AGPRs, operand fragments that fill half of the VGPRs): a vector register that spills lands in
+    scratch memory inside an MFMA chain and costs whole factors, which the numerics tests would not notice."""
+    out = {}
+    for m in re.finditer(r"- \.agpr_count:\s+\d+.*?\.wavefront_size", asm, re.S):
+        body = m.group(0)
+
+        def field(key, body=body):
+            mm = re.search(r"\." + key + r":\s+(\S+)", body)
+            return mm.group(1) if mm else None
+        name = field("name")
+        if name and name.startswith("_ZN2ma"):
+            out[name] = {"vgpr": int(field("vgpr_count")), "agpr": int(field("agpr_count")), "sgpr": int(field("sgpr_count")),
+                         "vgpr_spill": int(field("vgpr_spill_count")), "sgpr_spill": int(field("sgpr_spill_count")),
+                         "lds": int(field("group_segment_fixed_size"))}
+    return out
+
+
 def compile_to_assembly(source: str) -> str:
     with tempfile.TemporaryDirectory() as tmp:
         out = os.path.join(tmp, "k.s")
@@ -124,20 +144,26 @@ def compile_to_assembly(source: str) -> str:
             return f.read()
 
 
-def check_all(sources=SOURCES) -> tuple[list[str], dict]:
+def check_all(sources=SOURCES, resources: dict | None = None) -> tuple[list[str], dict]:
+    """Hazard check of every source; ``resources`` (a dict) is filled with ``kernel_resources`` of the same assembly."""
     bad, stats = [], {}
     with ThreadPoolExecutor(max_workers=len(sources)) as pool:
         for asm in pool.map(compile_to_assembly, sources):
             b, s = check_assembly(asm)
             bad += b
             stats.update(s)
+            if resources is not None:
+                resources.update(kernel_resources(asm))
     return bad, stats
 
 
 if __name__ == "__main__":
-    bad, stats = check_all(sys.argv[1:] or SOURCES)
+    res = {}
+    bad, stats = check_all(sys.argv[1:] or SOURCES, res)
     for name, (nm, ns) in stats.items():
-        print(f"{name}: {nm} asm MFMAs, {ns} asm scalar loads")
+        r = res.get(name, {})
+        print(f"{name}: {nm} asm MFMAs, {ns} asm scalar loads; {r.get('vgpr')} vector registers ({r.get('agpr')} of them accumulation), "
+              f"{r.get('vgpr_spill')} spilled; {r.get('sgpr_spill')} scalar registers spilled to vector lanes")
     for b in bad[:40]:
         print(b)
     print("BAD" if bad else "OK")

@@ -39,7 +39,8 @@ def test_checker_flags_every_kind_of_hazard():
 
 @pytest.mark.skipif(shutil.which("hipcc") is None, reason="hipcc not installed")
 def test_generated_assembly_of_the_attention_kernels_is_hazard_free():
-    bad, stats = isa_check.check_all()
+    res = {}
+    bad, stats = isa_check.check_all(resources=res)
     assert not bad, "\n".join(bad[:20])
     # every bf16 attention kernel went through the checker, and its asm MFMAs were seen
     # (three head dims x with / without document ids; the pair forward and the dK/dV kernel also with plain or
@@ -48,3 +49,14 @@ def test_generated_assembly_of_the_attention_kernels_is_hazard_free():
                           ("attn_bwd_dq_ds_bf16_kernel", 6), ("attn_bwd_dkv_bf16_kernel", 24)):
         hits = [v for k, v in stats.items() if kernel in k]
         assert len(hits) == count and all(n_mfma > 0 for n_mfma, _ in hits), (kernel, hits)
+    # The register budget the kernels are written around: no vector register of any bf16 attention kernel spills
+    # (a spill inside an MFMA chain costs whole factors and no numerics test would notice), the D = 256 kernels
+    # that hold two heads' accumulators use the whole file (all 256 accumulation registers), and the scalar
+    # registers spilled to vector lanes stay within what the step loops were tuned with.
+    attn = {k: v for k, v in res.items() if "attn_" in k and "bf16" in k}
+    assert len(attn) >= 60, len(attn)
+    assert all(v["vgpr_spill"] == 0 for v in attn.values()), {k: v["vgpr_spill"] for k, v in attn.items() if v["vgpr_spill"]}
+    assert all(v["sgpr_spill"] <= 80 for v in attn.values()), {k: v["sgpr_spill"] for k, v in attn.items() if v["sgpr_spill"] > 80}
+    for kernel in ("attn_fwd_pair_bf16_kernelILi256E", "attn_bwd_dkv_bf16_kernelILi256E", "attn_bwd_dq_ds_pair_bf16_kernelILi256E"):
+        hits = [v for k, v in attn.items() if kernel in k]
+        assert hits and all(v["agpr"] == 256 and v["vgpr"] <= 512 for v in hits), (kernel, hits)
